@@ -96,13 +96,15 @@ int hfa_attention_prompt_rows(void);
 // `force_plain`, runs the plain kernel. `slopes` (one fp32 per query head, or null) is the hook for a position
 // encoding that enters the scores rather than the queries and keys: the score of key j for the query at p
 // becomes dot * scale + slopes[h] * (j - p); with slopes the plain kernel runs. `sink` 1: the softmax has one more term
-// of score 0 that has no value, p_j = exp(s_j) / (1 + sum_i exp(s_i)) (every kernel takes it).
+// of score 0 that has no value, p_j = exp(s_j) / (1 + sum_i exp(s_i)) (every kernel takes it). `cross_values` 1: every
+// head's weights are applied to the values of every key/value group: out is [token][G rounds][H heads][v_head_dim], round r
+// of head h being its weights on the values of group (h's group + r) mod G (see hfa_talk_mix; the plain kernel runs).
 int hfa_paged_attention(const void* q, int dtype, int ldq, const void* k_cache, const void* v_cache,
                         int kv_width, int v_width, const int* block_table, int max_blocks, const int* token_slot,
                         const int* positions, const int* q_start, int n_seqs, int max_q_len, int max_seq_len,
                         void* out, int ldo, int n_tokens, int n_heads, int n_kv_heads, int head_dim, int v_head_dim,
-                        int page_tokens, int window, int mask_chunk, float scale, const float* slopes, int sink, void* workspace,
-                        size_t workspace_bytes, int force_plain, hipStream_t stream);
+                        int page_tokens, int window, int mask_chunk, float scale, const float* slopes, int sink, int cross_values,
+                        void* workspace, size_t workspace_bytes, int force_plain, hipStream_t stream);
 
 // Decoded tokens (one a request) whose queries, new keys and new values are still the 32-bit rows [q | k | v] that
 // the product left (`raw`, bias added): rotation of queries and keys (cos_sin: hfa_rope_table's output for the step's
@@ -129,10 +131,11 @@ int hfa_layernorm(float* x, const float* w, const float* b, void* out, int out_d
 
 // RMS norm in groups: a row of `width` values is cut into `groups` equal runs, each divided by sqrt(mean(run^2) + eps),
 // the whole times w; x and out fp32 or bf16, sums in fp32. rows: out[r] = norm(x[rows[r]]). gate_kind 1: the row is
-// multiplied by silu(gate[r]) before the norm; 2: the result is multiplied by sigmoid(gate[r]) (no rows then).
+// multiplied by silu(gate[r]) before the norm; 2: the result is multiplied by sigmoid(gate[r]) (no rows then). row_scale
+// (null: none; fp32 [n_rows, groups], rows in order): run g of row r is multiplied by row_scale[r, g] before everything else.
 int hfa_group_rmsnorm(const void* x, int x_dtype, int ldx, const float* w, void* out, int out_dtype, int ldo, const int* rows,
                       int n_rows, int width, int groups, float eps, const void* gate, int gate_dtype, int ldg, int gate_kind,
-                      hipStream_t stream);
+                      const float* row_scale, hipStream_t stream);
 
 // Rows [q: H D | k: G D | v: G Dv] of a step: optional RMS norm of the whole q part and of the whole k part (weights
 // q_norm_w, k_norm_w, eps), rotation of the first rot_dim dimensions of each q and k head (pairing 0: i with i + rot_dim / 2,
@@ -151,7 +154,15 @@ int hfa_qkv_prepare(void* qkv, int dtype, int ld, const int* positions, const fl
 // hfa_linear_scan: per head h (keys and queries of head h / (n_heads / qk_heads)), S [qk_dim][v_dim] in the state row (in the
 // kernel's own order, padded: hfa_linear_scan_state_floats values a row, zero for a new request; qk_dim at most 256):
 // S <- a_t S + k_t (b_t v_t)^T, y_t = S^T q_t + skip[h] v_t (skip null: 0). gate 0: a_t = decay[h], b_t = 1. gate 1:
-// dt = softplus(step[t, h] + step_bias[h]), a_t = exp(-exp(a_log[h]) dt), b_t = dt. y fp32.
+// dt = softplus(step[t, h] + step_bias[h]), a_t = exp(-exp(a_log[h]) dt), b_t = dt. y fp32. gate 2: exponential gates under a
+// running maximum m (kept beside the states): li = cap tanh((step + step_bias) / cap), lf = logsigmoid(cap tanh((step2 +
+// step_bias2) / cap)), m_t = max(lf + m, li), a_t = exp(lf + m - m_t), b_t = exp(li - m_t); the state has one more column that
+// holds n_t = a_t n + b_t k_t, and denom[t, h] = 1 / (max(|n_t . q_t|, exp(-m_t)) + 1e-6) leaves beside y (which is not divided).
+// A state row then holds hfa_linear_scan_state_floats(heads, qk_dim, v_dim + 1) + hfa_linear_scan_max_floats(...) values.
+// q_scale multiplies the queries.
+// hfa_delta_scan: the gated delta rule on fp32 inputs, S in hfa_linear_scan's layout: g_t[n] = exp(-exp(a_log[h]) softplus(a[t,
+// h N + n] + dt_bias[h N + n])), S <- g_t * S (row by row), u = sigmoid(b[t, h]) (v_t - S^T k_t), S <- S + k_t u^T, y_t = S^T q_t,
+// with k_t, q_t first divided by sqrt(sum of squares + unit_eps) and q_t multiplied by q_scale.
 int hfa_causal_conv(const void* in, int dtype, int ld_in, const float* taps, const float* bias, int n_channels, int n_taps,
                     float* state, size_t state_ld, const int* q_start, const int* seq_slot, int n_seqs, int max_q_len, float* out,
                     int ldo, int act, hipStream_t stream);
@@ -159,7 +170,35 @@ size_t hfa_linear_scan_state_floats(int n_heads, int qk_dim, int v_dim);
 int hfa_linear_scan(const void* q, int ldq, const void* k, int ldk, int qk_heads, int qk_dim, const void* v, int ldv, int n_heads,
                     int v_dim, int dtype, int gate, const float* decay, const void* step, int step_dtype, int ld_step,
                     const float* step_bias, const float* a_log, const float* skip, float* state, size_t state_ld,
-                    const int* q_start, const int* seq_slot, int n_seqs, float* y, int ldy, hipStream_t stream);
+                    const int* q_start, const int* seq_slot, int n_seqs, float* y, int ldy, const void* step2,
+                    const float* step_bias2, float cap, float q_scale, float* denom, hipStream_t stream);
+size_t hfa_linear_scan_max_floats(int n_heads, int qk_dim, int v_dim);
+int hfa_delta_scan(const float* q, int ldq, const float* k, int ldk, int qk_heads, int qk_dim, const float* v, int ldv, int n_heads,
+                   int v_dim, const float* a, int lda, const float* dt_bias, const float* a_log, const float* b, int ldb,
+                   float q_scale, float unit_eps, float* state, size_t state_ld, const int* q_start, const int* seq_slot,
+                   int n_seqs, float* y, int ldy, hipStream_t stream);
+
+// Layers that norm a branch's result before it joins the stream, and what comes with them (sandwich.hip).
+// hfa_embed_pos: x[t] = table[tokens[t]] * scale + pos(positions[t]), pos[2i] = sin(p inv_freq[i]), pos[2i + 1] = cos(p inv_freq[i])
+// (positions null: no position vector).
+// hfa_rmsnorm_add: v = y[r] * sigmoid(gate[r] + gate_bias) (gate null: v = y[r]); out[r] (+)= scale * v / sqrt(mean(v^2) + eps) * w.
+// hfa_polynorm: out = coef[0] N(z) + coef[1] N(z^2) + coef[2] N(z^3) + coef[3], N(u) = u / sqrt(mean(u^2) + eps) over a row.
+// hfa_scale_rows: x *= s. hfa_head_norm_store: rows [q | k | v]; q and k heads RMS-normed with a weight of one head's size (null:
+// as they are), q to q_out, k and v to cache rows slot_map[t] (values transposed inside their page).
+// hfa_talk_mix: out[t, h] = sigmoid(gate[t, h]) * sum_g talk[h, g] cross[t, (c(h) - c(g)) mod G, g], cross from hfa_paged_attention
+// with cross_values.
+int hfa_embed_pos(const void* table, int table_dtype, const int* tokens, const int* positions, const float* inv_freq, float* x,
+                  int n_tokens, int width, int vocab, float scale, hipStream_t stream);
+int hfa_rmsnorm_add(const float* y, int ldy, const void* gate, int gate_dtype, int ldg, const float* gate_bias, const float* w,
+                    float* out, int ldo, int n_rows, int width, float eps, float scale, int accumulate, hipStream_t stream);
+int hfa_polynorm(const void* z, int z_dtype, int ldz, const float* coef, void* out, int out_dtype, int ldo, int n_rows, int width,
+                 float eps, hipStream_t stream);
+int hfa_scale_rows(float* x, int ld, int n_rows, int width, float s, hipStream_t stream);
+int hfa_head_norm_store(const void* qkv, int in_dtype, int ld, int n_heads, int n_kv_heads, int head_dim, int v_head_dim,
+                        const float* q_w, const float* k_w, float eps, void* q_out, int ldq, void* k_cache, void* v_cache,
+                        int out_dtype, const int* slot_map, int page_tokens, int n_tokens, hipStream_t stream);
+int hfa_talk_mix(const void* cross, int cross_dtype, const float* talk, const void* gate, int gate_dtype, int ldg, void* out,
+                 int out_dtype, int ldo, int n_tokens, int n_heads, int n_kv_heads, int v_head_dim, hipStream_t stream);
 
 // out[r, c] = act(in[r, c]) for rows of `width` values with strides ldi and ldo, computed in fp32:
 // the exact gelu 0.5 z (1 + erf(z / sqrt 2)), its tanh form, relu(z)^2, silu or the logistic function.

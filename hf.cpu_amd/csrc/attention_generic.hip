@@ -42,7 +42,11 @@ __device__ __forceinline__ float dot_row(const float* __restrict__ q_s, const fl
     return dot;
 }
 
-template <typename T>
+// CROSS: every query head's weights are applied to the values of EVERY key/value group (the whole value row, up to
+// ATT_MAX_CROSS columns), and out is [token][G rounds][H heads][Dv]: round r of head h holds its weights on the values of
+// group (h's group + r) mod G. A design that mixes the heads' weights after the softmax sums these (hfa_talk_mix).
+#define ATT_MAX_CROSS 1024
+template <typename T, bool CROSS>
 __global__ __launch_bounds__(WAVE) void attn_generic_kernel(
     const T* __restrict__ q, int ldq, const T* __restrict__ kc, const T* __restrict__ vc, int kvw, int vw,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_slot,
@@ -60,9 +64,11 @@ __global__ __launch_bounds__(WAVE) void attn_generic_kernel(
     const int lo = first_visible(pos, window, mask_chunk);
     const float slope = slopes ? slopes[h] : 0.f;           // a position encoding that enters the scores
     float m = -INFINITY, l = 0.f;
-    float acc[ATT_MAX_D / WAVE];
+    constexpr int NACC = (CROSS ? ATT_MAX_CROSS : ATT_MAX_D) / WAVE;
+    const int v_first = CROSS ? 0 : kvh * Dv, v_cols = CROSS ? G * Dv : Dv;      // the columns of a value row that this head reads
+    float acc[NACC];
 #pragma unroll
-    for (int i = 0; i < ATT_MAX_D / WAVE; i++) acc[i] = 0.f;
+    for (int i = 0; i < NACC; i++) acc[i] = 0.f;
 
     for (int j0 = (lo / WAVE) * WAVE; j0 <= pos; j0 += WAVE) {
         const int j = j0 + lane;
@@ -86,45 +92,52 @@ __global__ __launch_bounds__(WAVE) void attn_generic_kernel(
         const int first = lo > j0 ? lo - j0 : 0;
         const int last = pos - j0 < WAVE - 1 ? pos - j0 : WAVE - 1;
 #pragma unroll
-        for (int i = 0; i < ATT_MAX_D / WAVE; i++) acc[i] *= corr;
+        for (int i = 0; i < NACC; i++) acc[i] *= corr;
         for (int jj = first; jj <= last; jj++) {
             const float pj = p_s[jj];
             // values lie transposed inside their page: [page][column][token]
             const int vr = row_s[jj];
-            const T* vp = vc + (size_t)(vr / page_tokens) * page_tokens * vw + (size_t)(kvh * Dv) * page_tokens +
+            const T* vp = vc + (size_t)(vr / page_tokens) * page_tokens * vw + (size_t)v_first * page_tokens +
                           vr % page_tokens;
 #pragma unroll
-            for (int i = 0; i < ATT_MAX_D / WAVE; i++) {
+            for (int i = 0; i < NACC; i++) {
                 const int d = lane + WAVE * i;
-                if (d < Dv) acc[i] = fmaf(pj, to_f32(vp[(size_t)d * page_tokens]), acc[i]);
+                if (d < v_cols) acc[i] = fmaf(pj, to_f32(vp[(size_t)d * page_tokens]), acc[i]);
             }
         }
         __syncthreads();
     }
     const float inv = 1.0f / (sink ? l + expf(-m) : l);      // the term of score 0 that has no value
 #pragma unroll
-    for (int i = 0; i < ATT_MAX_D / WAVE; i++) {
+    for (int i = 0; i < NACC; i++) {
         const int d = lane + WAVE * i;
-        if (d < Dv) out[(size_t)t * ldo + h * Dv + d] = from_f32<T>(acc[i] * inv);
+        if (d >= v_cols) continue;
+        if (CROSS) {
+            const int vh = d / Dv, r = (vh - kvh + G) % G;
+            out[(size_t)t * ldo + ((size_t)r * H + h) * Dv + d % Dv] = from_f32<T>(acc[i] * inv);
+        } else {
+            out[(size_t)t * ldo + h * Dv + d] = from_f32<T>(acc[i] * inv);
+        }
     }
 }
 
 int attn_generic_launch(const void* q, int dtype, int ldq, const void* k_cache, const void* v_cache, int kv_width,
                         int v_width, const int* block_table, int max_blocks, const int* token_slot, const int* positions,
                         void* out, int ldo, int n_tokens, int n_heads, int n_kv_heads, int head_dim, int v_head_dim,
-                        int page_tokens, int window, int mask_chunk, float scale, const float* slopes, int sink, hipStream_t stream) {
+                        int page_tokens, int window, int mask_chunk, float scale, const float* slopes, int sink, int cross, hipStream_t stream) {
+    HFA_REQUIRE(!cross || n_kv_heads * v_head_dim <= ATT_MAX_CROSS, "paged_attention: a value row of %d columns exceeds what one wave "
+                "applies its weights to (%d)", n_kv_heads * v_head_dim, ATT_MAX_CROSS);
     HFA_REQUIRE(head_dim <= ATT_MAX_D && v_head_dim <= ATT_MAX_D, "paged_attention: head_dim %d (values: %d) exceeds the kernel's limit %d",
                 head_dim, v_head_dim, ATT_MAX_D);
     HFA_REQUIRE(n_heads <= 65535, "paged_attention: %d heads exceed the grid", n_heads);
     dim3 grid(n_tokens, n_heads);
-    if (dtype == HFA_F32)
-        attn_generic_kernel<float><<<grid, WAVE, 0, stream>>>(
-            (const float*)q, ldq, (const float*)k_cache, (const float*)v_cache, kv_width, v_width, block_table, max_blocks,
-            token_slot, positions, (float*)out, ldo, n_heads, n_kv_heads, head_dim, v_head_dim, page_tokens, window, mask_chunk, scale, slopes, sink);
-    else
-        attn_generic_kernel<bf16><<<grid, WAVE, 0, stream>>>(
-            (const bf16*)q, ldq, (const bf16*)k_cache, (const bf16*)v_cache, kv_width, v_width, block_table, max_blocks,
-            token_slot, positions, (bf16*)out, ldo, n_heads, n_kv_heads, head_dim, v_head_dim, page_tokens, window, mask_chunk, scale, slopes, sink);
+#define ATT_GO(T, CROSS)                                                                                                          \
+    attn_generic_kernel<T, CROSS><<<grid, WAVE, 0, stream>>>(                                                                     \
+        (const T*)q, ldq, (const T*)k_cache, (const T*)v_cache, kv_width, v_width, block_table, max_blocks, token_slot, positions, \
+        (T*)out, ldo, n_heads, n_kv_heads, head_dim, v_head_dim, page_tokens, window, mask_chunk, scale, slopes, sink)
+    if (dtype == HFA_F32) { if (cross) ATT_GO(float, true); else ATT_GO(float, false); }
+    else { if (cross) ATT_GO(bf16, true); else ATT_GO(bf16, false); }
+#undef ATT_GO
     HFA_LAUNCH_CHECK("paged_attention");
     return 0;
 }
@@ -191,14 +204,14 @@ extern "C" int hfa_paged_attention(const void* q, int dtype, int ldq, const void
                                    const int* positions, const int* q_start, int n_seqs, int max_q_len,
                                    int max_seq_len, void* out, int ldo, int n_tokens, int n_heads, int n_kv_heads,
                                    int head_dim, int v_head_dim, int page_tokens, int window, int mask_chunk, float scale,
-                                   const float* slopes, int sink, void* workspace, size_t workspace_bytes, int force_plain,
-                                   hipStream_t stream) {
+                                   const float* slopes, int sink, int cross_values, void* workspace, size_t workspace_bytes,
+                                   int force_plain, hipStream_t stream) {
     HFA_REQUIRE(n_tokens > 0 && n_heads > 0 && n_kv_heads > 0 && head_dim > 0 && v_head_dim > 0 && page_tokens > 0 && max_blocks > 0,
                 "paged_attention: bad sizes");
     HFA_REQUIRE(n_heads % n_kv_heads == 0, "paged_attention: %d heads are not a multiple of %d key/value heads",
                 n_heads, n_kv_heads);
     HFA_REQUIRE(kv_width >= n_kv_heads * head_dim && v_width >= n_kv_heads * v_head_dim && ldq >= n_heads * head_dim &&
-                    ldo >= n_heads * v_head_dim,
+                    ldo >= n_heads * v_head_dim * (cross_values ? n_kv_heads : 1),
                 "paged_attention: a row stride is smaller than its row");
     HFA_REQUIRE(window >= 0 && mask_chunk >= 0, "paged_attention: negative window or masking chunk");
     HFA_REQUIRE(dtype == HFA_F32 || dtype == HFA_BF16, "paged_attention: unknown dtype %d", dtype);
@@ -207,9 +220,9 @@ extern "C" int hfa_paged_attention(const void* q, int dtype, int ldq, const void
                   window, scale, workspace, workspace_bytes, stream, nullptr, 0, nullptr, nullptr, mask_chunk, sink ? 1 : 0};
     // the matrix-core kernels take no slopes: scores with a position term go the plain way
     // and they know one head size and one row width for keys and values
-    if (!force_plain && !slopes && dtype == HFA_BF16 && v_head_dim == head_dim && v_width == kv_width && attn_mfma_supports(a))
+    if (!force_plain && !slopes && !cross_values && dtype == HFA_BF16 && v_head_dim == head_dim && v_width == kv_width && attn_mfma_supports(a))
         return attn_mfma_launch(a);
     return attn_generic_launch(q, dtype, ldq, k_cache, v_cache, kv_width, v_width, block_table, max_blocks, token_slot,
                                positions, out, ldo, n_tokens, n_heads, n_kv_heads, head_dim, v_head_dim, page_tokens, window,
-                               mask_chunk, scale, slopes, sink ? 1 : 0, stream);
+                               mask_chunk, scale, slopes, sink ? 1 : 0, cross_values ? 1 : 0, stream);
 }

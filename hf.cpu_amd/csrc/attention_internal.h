@@ -36,7 +36,7 @@ __host__ __device__ __forceinline__ int first_visible(int pos, int window, int m
 int attn_generic_launch(const void* q, int dtype, int ldq, const void* k_cache, const void* v_cache, int kv_width,
                         int v_width, const int* block_table, int max_blocks, const int* token_slot, const int* positions,
                         void* out, int ldo, int n_tokens, int n_heads, int n_kv_heads, int head_dim, int v_head_dim,
-                        int page_tokens, int window, int mask_chunk, float scale, const float* slopes, int sink, hipStream_t stream);
+                        int page_tokens, int window, int mask_chunk, float scale, const float* slopes, int sink, int cross, hipStream_t stream);
 
 // bf16 on the matrix cores; see attention_mfma.hip for what it needs.
 bool attn_mfma_supports(const AttnArgs& a);

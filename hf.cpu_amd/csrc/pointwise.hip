@@ -140,15 +140,16 @@ template <typename TX, typename TG, typename TO>
 __global__ __launch_bounds__(1024) void group_rmsnorm_kernel(const TX* __restrict__ x, int ldx, const float* __restrict__ w,
                                                             TO* __restrict__ out, int ldo, const int* __restrict__ rows,
                                                             int run, float eps, const TG* __restrict__ gate, int ldg,
-                                                            int gate_kind) {
+                                                            int gate_kind, const float* __restrict__ row_scale) {
     __shared__ float red[17];
     const int r = blockIdx.x, c0 = blockIdx.y * run;
+    const float pre = row_scale ? row_scale[(size_t)r * gridDim.y + blockIdx.y] : 1.f;     // a factor of this (row, run), before the norm
     const TX* src = x + (size_t)(rows ? rows[r] : r) * ldx + c0;
     const TG* gsrc = gate ? gate + (size_t)r * ldg + c0 : nullptr;
     constexpr int KEEP = 4;
     float keep[KEEP];
     auto value = [&](int i) {
-        float v = to_f32(src[i]);
+        float v = to_f32(src[i]) * pre;
         if (gate_kind == 1) {
             const float z = to_f32(gsrc[i]);
             v *= z / (1.0f + expf(-z));
@@ -183,7 +184,8 @@ __global__ __launch_bounds__(1024) void group_rmsnorm_kernel(const TX* __restric
 
 extern "C" int hfa_group_rmsnorm(const void* x, int x_dtype, int ldx, const float* w, void* out, int out_dtype, int ldo,
                                  const int* rows, int n_rows, int width, int groups, float eps, const void* gate,
-                                 int gate_dtype, int ldg, int gate_kind, hipStream_t stream) {
+                                 int gate_dtype, int ldg, int gate_kind, const float* row_scale, hipStream_t stream) {
+    HFA_REQUIRE(!row_scale || !rows, "group_rmsnorm: factors per (row, run) go with rows in order");
     HFA_REQUIRE(x && w && out && n_rows > 0 && width > 0 && ldx >= width && ldo >= width, "group_rmsnorm: bad arguments");
     HFA_REQUIRE(groups > 0 && width % groups == 0 && groups <= 65535, "group_rmsnorm: %d values do not form %d equal runs", width, groups);
     HFA_REQUIRE((x_dtype == HFA_F32 || x_dtype == HFA_BF16) && (out_dtype == HFA_F32 || out_dtype == HFA_BF16),
@@ -196,7 +198,7 @@ extern "C" int hfa_group_rmsnorm(const void* x, int x_dtype, int ldx, const floa
     dim3 grid(n_rows, groups);
 #define GRN(TX, TG, TO)                                                                                                 \
     group_rmsnorm_kernel<TX, TG, TO><<<grid, threads, 0, stream>>>((const TX*)x, ldx, w, (TO*)out, ldo, rows, run, eps, \
-                                                                   (const TG*)(gate_kind ? gate : nullptr), ldg, gate_kind)
+                                                                   (const TG*)(gate_kind ? gate : nullptr), ldg, gate_kind, row_scale)
     const bool gb = gate_kind && gate_dtype == HFA_BF16;
     if (x_dtype == HFA_F32 && out_dtype == HFA_F32) { if (gb) GRN(float, bf16, float); else GRN(float, float, float); }
     else if (x_dtype == HFA_F32) { if (gb) GRN(float, bf16, bf16); else GRN(float, float, bf16); }

@@ -5,6 +5,7 @@
 //                     before a request's first token of this step taken from its state row, which then receives the
 //                     last K - 1 inputs of the step
 //   hfa_linear_scan   S <- a_t S + k_t (b_t v_t)^T, y_t = S^T q_t + d v_t per (request, head), S in fp32 in the state row
+//   hfa_delta_scan    S <- g_t * S (a decay per row), u = beta_t (v_t - S^T k_t), S <- S + k_t u^T, y_t = S^T q_t
 //
 // Both walk a request's tokens of the step in order from the state that the step before left, so a token's result
 // does not depend on where a prompt was cut or on what else the step holds.
@@ -95,6 +96,13 @@ extern "C" int hfa_causal_conv(const void* in, int dtype, int ld_in, const float
 //
 // gate 0: a_t = decay[h], b_t = 1 (a fixed decay per head).
 // gate 1: dt = softplus(step[t, h] + step_bias[h]), a_t = exp(-exp(a_log[h]) dt), b_t = dt (a step size per token).
+// gate 2: exponential gates kept stable by a running maximum m (0 for a new request, kept beside the states): with
+//         li = cap tanh((step[t, h] + step_bias[h]) / cap) and lf = logsigmoid(cap tanh((step2[t, h] + step_bias2[h]) / cap)),
+//         m_t = max(lf + m_(t-1), li), a_t = exp(lf + m_(t-1) - m_t), b_t = exp(li - m_t). The state has one more column
+//         whose value is 1 for every token, so that it holds n_t = a_t n_(t-1) + b_t k_t; its output n_t . q_t does not
+//         leave as a column of y but as denom[t, h] = 1 / (max(|n_t . q_t|, exp(-m_t)) + 1e-6), by which the reader of y
+//         multiplies the head's outputs. Every block of columns keeps a copy of m of its own (a block may start after
+//         another of the same head has ended), behind the states: m_off + h * blocks + block.
 #define SCAN_TOKENS 16
 #define SCAN_THREADS 256
 
@@ -120,14 +128,15 @@ __global__ __launch_bounds__(SCAN_THREADS) void linear_scan_kernel(
     int ldv, int P, int gate, const float* __restrict__ decay, const TS* __restrict__ step, int ld_step,
     const float* __restrict__ step_bias, const float* __restrict__ a_log, const float* __restrict__ skip,
     float* __restrict__ state, size_t state_ld, const int* __restrict__ q_start, const int* __restrict__ seq_slot,
-    float* __restrict__ y, int ldy) {
+    float* __restrict__ y, int ldy, const TS* __restrict__ step2, const float* __restrict__ step_bias2, float cap, float q_scale,
+    float* __restrict__ denom, size_t m_off) {
     constexpr int NPAD = NS * NPT, PT = SCAN_THREADS / NS, TOK = SCAN_TOKENS;
     constexpr int RK = TOK * NPAD / SCAN_THREADS, RV = (TOK * PT + SCAN_THREADS - 1) / SCAN_THREADS;
     static_assert(TOK * NPAD % SCAN_THREADS == 0 && NPT % 4 == 0, "the staging loops are whole");
     __shared__ __attribute__((aligned(16))) float k_s[TOK * NPAD];
     __shared__ __attribute__((aligned(16))) float q_s[TOK * NPAD];
     __shared__ float v_s[TOK * PT];
-    __shared__ float a_s[TOK], b_s[TOK];
+    __shared__ float a_s[TOK], b_s[TOK], m_s[TOK];
     __shared__ __attribute__((aligned(16))) float part_s[TOK * SCAN_THREADS];      // [token][column][lane of the column]
     const int h = blockIdx.x, s = blockIdx.y, pz = blockIdx.z, tid = threadIdx.x;
     const int pl = tid / NS, ns = tid % NS;
@@ -140,13 +149,16 @@ __global__ __launch_bounds__(SCAN_THREADS) void linear_scan_kernel(
     for (int i = 0; i < NPT; i++) st[i] = S[(size_t)i * p_pad * NS];
     const float d = skip ? skip[h] : 0.f;
     const float head_decay = gate == 0 ? decay[h] : 0.f;
-    const float neg_rate = gate == 1 ? -expf(a_log[h]) : 0.f, sb = gate == 1 ? step_bias[h] : 0.f;
+    const float neg_rate = gate == 1 ? -expf(a_log[h]) : 0.f, sb = gate >= 1 ? step_bias[h] : 0.f;
+    const float sb2 = gate == 2 ? step_bias2[h] : 0.f, inv_cap = gate == 2 ? 1.0f / cap : 0.f;
+    float* m_at = state + (size_t)seq_slot[s] * state_ld + m_off + (size_t)h * gridDim.z + pz;
+    float m_run = gate == 2 ? *m_at : 0.f;               // the running maximum, followed by the block's first wave
     const T* kg = k + (size_t)q0 * ldk + g * N;
     const T* qg = q + (size_t)q0 * ldq + g * N;
     const T* vg = v + (size_t)q0 * ldv + h * P + pz * PT;
     // Two sets of registers take turns: while one chunk of tokens is walked, the loads of the next two are on their way
     // (a trip to memory takes longer than the walk of one chunk).
-    struct Staged { float k[RK], q[RK], v[RV], step; };
+    struct Staged { float k[RK], q[RK], v[RV], step, step2; };
     Staged set_a, set_b;
     // the tokens c0 .. c0 + TOK - 1 into registers (zeros beyond the request's tokens, beyond N and beyond P)
     auto fetch = [&](Staged& g_, int c0) {
@@ -162,19 +174,34 @@ __global__ __launch_bounds__(SCAN_THREADS) void linear_scan_kernel(
         for (int r = 0; r < RV; r++) {
             const int idx = tid + r * SCAN_THREADS, t = c0 + idx / PT, pp = idx % PT;
             g_.v[r] = (idx < TOK * PT && t < n_tok && pz * PT + pp < P) ? to_f32(vg[(size_t)t * ldv + pp]) : 0.f;
+            if (gate == 2 && idx < TOK * PT && t < n_tok && pz * PT + pp == P) g_.v[r] = 1.f;       // the normaliser's column
         }
-        g_.step = (gate == 1 && tid < TOK && c0 + tid < n_tok) ? to_f32(step[(size_t)(q0 + c0 + tid) * ld_step + h]) : 0.f;
+        g_.step = (gate >= 1 && tid < TOK && c0 + tid < n_tok) ? to_f32(step[(size_t)(q0 + c0 + tid) * ld_step + h]) : 0.f;
+        g_.step2 = (gate == 2 && tid < TOK && c0 + tid < n_tok) ? to_f32(step2[(size_t)(q0 + c0 + tid) * ld_step + h]) : 0.f;
     };
-    auto stash = [&](const Staged& g_) {
+    auto stash = [&](const Staged& g_, int c0) {
 #pragma unroll
         for (int r = 0; r < RK; r++) {
             k_s[tid + r * SCAN_THREADS] = g_.k[r];
-            q_s[tid + r * SCAN_THREADS] = g_.q[r];
+            q_s[tid + r * SCAN_THREADS] = g_.q[r] * q_scale;
         }
 #pragma unroll
         for (int r = 0; r < RV; r++)
             if (tid + r * SCAN_THREADS < TOK * PT) v_s[tid + r * SCAN_THREADS] = g_.v[r];
-        if (tid < TOK) {
+        if (gate == 2) {
+            if (tid < WAVE) {                                   // the maximum runs from token to token: one wave, in order
+                const float li = cap * tanhf((g_.step + sb) * inv_cap), zf = cap * tanhf((g_.step2 + sb2) * inv_cap);
+                const float lf = -(fmaxf(-zf, 0.f) + log1pf(expf(-fabsf(zf))));          // logsigmoid
+                float a_mine = 0.f, b_mine = 0.f, m_mine = 0.f;
+                for (int t = 0; t < TOK && c0 + t < n_tok; t++) {
+                    const float f_t = __shfl(lf, t, WAVE), i_t = __shfl(li, t, WAVE);
+                    const float mn = fmaxf(f_t + m_run, i_t);
+                    if (tid == t) { a_mine = expf(f_t + m_run - mn); b_mine = expf(i_t - mn); m_mine = mn; }
+                    m_run = mn;
+                }
+                if (tid < TOK) { a_s[tid] = a_mine; b_s[tid] = b_mine; m_s[tid] = m_mine; }
+            }
+        } else if (tid < TOK) {
             if (gate == 1) {
                 const float z = g_.step + sb;
                 const float dt = fmaxf(z, 0.f) + log1pf(expf(-fabsf(z)));          // softplus, exact for every z
@@ -189,7 +216,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void linear_scan_kernel(
     auto chunk = [&](Staged& g_, int c0) {
         const int nt = n_tok - c0 < TOK ? n_tok - c0 : TOK;
         __syncthreads();                                   // the walk before has read what is overwritten now
-        stash(g_);
+        stash(g_, c0);
         __syncthreads();
         fetch(g_, c0 + 2 * TOK);
         // A token's operands leave LDS two tokens before (three gained nothing) its multiply-adds: the only chain from token to token is the
@@ -242,7 +269,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void linear_scan_kernel(
         // the outputs of the tokens just walked: thread -> (token, column), the lanes' shares added in lane order
         for (int idx = tid; idx < nt * PT; idx += SCAN_THREADS) {
             const int t = idx / PT, pp = idx % PT;
-            if (pz * PT + pp >= P) continue;
+            if (pz * PT + pp > P || (pz * PT + pp == P && gate != 2)) continue;
             const float4* sh = reinterpret_cast<const float4*>(part_s + t * SCAN_THREADS + pp * NS);
             float acc = 0.f;
 #pragma unroll
@@ -250,7 +277,228 @@ __global__ __launch_bounds__(SCAN_THREADS) void linear_scan_kernel(
                 const float4 u = sh[i];
                 acc = ((acc + u.x) + u.y) + u.z + u.w;
             }
-            y[(size_t)(q0 + c0 + t) * ldy + h * P + pz * PT + pp] = fmaf(d, v_s[t * PT + pp], acc);
+            if (pz * PT + pp == P)
+                denom[(size_t)(q0 + c0 + t) * gridDim.x + h] = 1.0f / (fmaxf(fabsf(acc), expf(-m_s[t])) + 1e-6f);
+            else
+                y[(size_t)(q0 + c0 + t) * ldy + h * P + pz * PT + pp] = fmaf(d, v_s[t * PT + pp], acc);
+        }
+    };
+    fetch(set_a, 0);
+    fetch(set_b, TOK);
+    for (int c0 = 0; c0 < n_tok; c0 += 2 * TOK) {
+        chunk(set_a, c0);
+        if (c0 + TOK < n_tok) chunk(set_b, c0 + TOK);
+    }
+#pragma unroll
+    for (int i = 0; i < NPT; i++) S[(size_t)i * p_pad * NS] = st[i];
+    if (gate == 2 && tid == 0) *m_at = m_run;
+}
+
+extern "C" size_t hfa_linear_scan_max_floats(int n_heads, int qk_dim, int v_dim) {
+    int ns, npt;
+    scan_shape(qk_dim, &ns, &npt);
+    const int pt = SCAN_THREADS / ns;
+    return (size_t)n_heads * ((v_dim + 1 + pt - 1) / pt);
+}
+
+extern "C" int hfa_linear_scan(const void* q, int ldq, const void* k, int ldk, int qk_heads, int qk_dim, const void* v,
+                               int ldv, int n_heads, int v_dim, int dtype, int gate, const float* decay, const void* step,
+                               int step_dtype, int ld_step, const float* step_bias, const float* a_log, const float* skip,
+                               float* state, size_t state_ld, const int* q_start, const int* seq_slot, int n_seqs, float* y,
+                               int ldy, const void* step2, const float* step_bias2, float cap, float q_scale, float* denom,
+                               hipStream_t stream) {
+    HFA_REQUIRE(q && k && v && state && q_start && seq_slot && y && n_seqs > 0, "linear_scan: a null argument");
+    HFA_REQUIRE(n_heads > 0 && qk_heads > 0 && n_heads % qk_heads == 0 && qk_dim > 0 && v_dim > 0,
+                "linear_scan: %d heads over %d heads of keys", n_heads, qk_heads);
+    HFA_REQUIRE(qk_dim <= 256, "linear_scan: a state of %d rows a head is too large (at most 256)", qk_dim);
+    HFA_REQUIRE(ldq >= qk_heads * qk_dim && ldk >= qk_heads * qk_dim && ldv >= n_heads * v_dim && ldy >= n_heads * v_dim &&
+                    state_ld >= hfa_linear_scan_state_floats(n_heads, qk_dim, v_dim + (gate == 2 ? 1 : 0)) +
+                                    (gate == 2 ? hfa_linear_scan_max_floats(n_heads, qk_dim, v_dim) : 0),
+                "linear_scan: a row is shorter than its heads (a state row holds hfa_linear_scan_state_floats values; gate 2: "
+                "those of one more column, and hfa_linear_scan_max_floats)");
+    HFA_REQUIRE(dtype == HFA_F32 || dtype == HFA_BF16, "linear_scan: unknown dtype %d", dtype);
+    HFA_REQUIRE((gate == 0 && decay) || (gate == 1 && step && step_bias && a_log && ld_step >= n_heads &&
+                                         (step_dtype == HFA_F32 || step_dtype == HFA_BF16)) ||
+                    (gate == 2 && step && step2 && step_bias && step_bias2 && denom && cap > 0.f && !skip && ld_step >= n_heads &&
+                     (step_dtype == HFA_F32 || step_dtype == HFA_BF16)),
+                "linear_scan: gate 0 needs a decay per head, gate 1 step sizes, their bias and the logarithm of the rate, gate 2 "
+                "both gates' inputs and biases, a positive cap and a place for the denominators (and no skip)");
+    int ns, npt;
+    scan_shape(qk_dim, &ns, &npt);
+    const int pt = SCAN_THREADS / ns, p_tiles = (v_dim + (gate == 2 ? 1 : 0) + pt - 1) / pt;
+    const size_t m_off = hfa_linear_scan_state_floats(n_heads, qk_dim, v_dim + 1);
+    HFA_REQUIRE(n_heads <= 65535 && n_seqs <= 65535 && p_tiles <= 65535, "linear_scan: the step exceeds the grid");
+    dim3 grid(n_heads, n_seqs, p_tiles);
+#define SCAN_GO(T, TS, NS, NPT)                                                                                          \
+    linear_scan_kernel<T, TS, NS, NPT><<<grid, SCAN_THREADS, 0, stream>>>(                                               \
+        (const T*)q, ldq, (const T*)k, ldk, n_heads / qk_heads, qk_dim, (const T*)v, ldv, v_dim, gate, decay, (const TS*)step, \
+        ld_step, step_bias, a_log, skip, state, state_ld, q_start, seq_slot, y, ldy, (const TS*)step2, step_bias2, cap, q_scale, \
+        denom, m_off)
+#define SCAN_SIZES(T, TS)                                          \
+    do {                                                           \
+        if (ns == 4) SCAN_GO(T, TS, 4, 4);                         \
+        else if (ns == 8 && npt == 4) SCAN_GO(T, TS, 8, 4);        \
+        else if (ns == 8) SCAN_GO(T, TS, 8, 8);                    \
+        else if (npt == 4) SCAN_GO(T, TS, 16, 4);                  \
+        else if (npt == 8) SCAN_GO(T, TS, 16, 8);                  \
+        else SCAN_GO(T, TS, 16, 16);                               \
+    } while (0)
+    if (dtype == HFA_F32) { if (step_dtype == HFA_BF16 && gate >= 1) SCAN_SIZES(float, bf16); else SCAN_SIZES(float, float); }
+    else { if (step_dtype == HFA_F32 && gate >= 1) SCAN_SIZES(bf16, float); else SCAN_SIZES(bf16, bf16); }
+#undef SCAN_SIZES
+#undef SCAN_GO
+    HFA_LAUNCH_CHECK("linear_scan");
+    return 0;
+}
+
+// ---- the gated delta rule ----------------------------------------------------------------------------------------------
+// Per head h (queries and keys of head h / (n_heads / qk_heads)), S [N][P] in the state row, in hfa_linear_scan's layout:
+//   g_t[n] = exp(-exp(a_log[h]) softplus(a[t, h N + n] + dt_bias[h N + n]))        a decay per key channel (row of S)
+//   S <- g_t * S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T;  y_t = S^T q_t     beta_t = sigmoid(b[t, h])
+// with k_t and q_t made unit vectors first (x / sqrt(sum x^2 + unit_eps)) and q_t times q_scale. All inputs, the state
+// and every operation are fp32. The block, its lanes and the staging through LDS are linear_scan_kernel's; what differs is
+// that a token's correction needs S^T k_t whole before the state moves, so the lanes of a column add their shares of it
+// across lanes inside the walk (a butterfly: every lane gets the same bits), where that kernel has no traffic at all.
+template <int NS, int NPT>
+__global__ __launch_bounds__(SCAN_THREADS) void delta_scan_kernel(
+    const float* __restrict__ q, int ldq, const float* __restrict__ k, int ldk, int heads_per_qk, int N, const float* __restrict__ v,
+    int ldv, int P, const float* __restrict__ a, int lda, const float* __restrict__ dt_bias, const float* __restrict__ a_log,
+    const float* __restrict__ b, int ldb, float q_scale, float unit_eps, float* __restrict__ state, size_t state_ld,
+    const int* __restrict__ q_start, const int* __restrict__ seq_slot, float* __restrict__ y, int ldy) {
+    constexpr int NPAD = NS * NPT, PT = SCAN_THREADS / NS, TOK = SCAN_TOKENS;
+    constexpr int RK = TOK * NPAD / SCAN_THREADS, RV = (TOK * PT + SCAN_THREADS - 1) / SCAN_THREADS;
+    static_assert(TOK * NPAD % SCAN_THREADS == 0 && NPT % 4 == 0, "the staging loops are whole");
+    __shared__ __attribute__((aligned(16))) float k_s[TOK * NPAD];
+    __shared__ __attribute__((aligned(16))) float q_s[TOK * NPAD];
+    __shared__ __attribute__((aligned(16))) float g_s[TOK * NPAD];
+    __shared__ float v_s[TOK * PT];
+    __shared__ float b_s[TOK];
+    __shared__ __attribute__((aligned(16))) float part_s[TOK * SCAN_THREADS];
+    const int h = blockIdx.x, s = blockIdx.y, pz = blockIdx.z, tid = threadIdx.x;
+    const int pl = tid / NS, ns = tid % NS, lane = tid & (WAVE - 1), wv = tid / WAVE;
+    const int q0 = q_start[s], n_tok = q_start[s + 1] - q0;
+    if (n_tok <= 0) return;
+    const int g = h / heads_per_qk, p_pad = (int)gridDim.z * PT;
+    float* S = state + (size_t)seq_slot[s] * state_ld + (size_t)h * NPT * p_pad * NS + (size_t)pz * SCAN_THREADS + tid;
+    float st[NPT];
+#pragma unroll
+    for (int i = 0; i < NPT; i++) st[i] = S[(size_t)i * p_pad * NS];
+    const float neg_rate = -expf(a_log[h]);
+    const float* kg = k + (size_t)q0 * ldk + g * N;
+    const float* qg = q + (size_t)q0 * ldq + g * N;
+    const float* ag = a + (size_t)q0 * lda + h * N;
+    const float* vg = v + (size_t)q0 * ldv + h * P + pz * PT;
+    float bias_r[RK];                                      // the decay's bias of the channels this thread stages
+#pragma unroll
+    for (int r = 0; r < RK; r++) {
+        const int n = (tid + r * SCAN_THREADS) % NPAD;
+        bias_r[r] = n < N ? dt_bias[h * N + n] : 0.f;
+    }
+    struct Staged { float k[RK], q[RK], a[RK], v[RV], b; };
+    Staged set_a, set_b;
+    auto fetch = [&](Staged& g_, int c0) {
+        if (c0 >= n_tok) return;
+#pragma unroll
+        for (int r = 0; r < RK; r++) {
+            const int idx = tid + r * SCAN_THREADS, t = c0 + idx / NPAD, n = idx % NPAD;
+            const bool ok = t < n_tok && n < N;
+            g_.k[r] = ok ? kg[(size_t)t * ldk + n] : 0.f;
+            g_.q[r] = ok ? qg[(size_t)t * ldq + n] : 0.f;
+            g_.a[r] = ok ? ag[(size_t)t * lda + n] : 0.f;
+        }
+#pragma unroll
+        for (int r = 0; r < RV; r++) {
+            const int idx = tid + r * SCAN_THREADS, t = c0 + idx / PT, pp = idx % PT;
+            g_.v[r] = (idx < TOK * PT && t < n_tok && pz * PT + pp < P) ? vg[(size_t)t * ldv + pp] : 0.f;
+        }
+        g_.b = (tid < TOK && c0 + tid < n_tok) ? b[(size_t)(q0 + c0 + tid) * ldb + h] : 0.f;
+    };
+    auto stash = [&](const Staged& g_) {
+#pragma unroll
+        for (int r = 0; r < RK; r++) {
+            const int idx = tid + r * SCAN_THREADS;
+            k_s[idx] = g_.k[r];
+            q_s[idx] = g_.q[r];
+            const float z = g_.a[r] + bias_r[r];
+            const float sp = fmaxf(z, 0.f) + log1pf(expf(-fabsf(z)));                 // softplus, exact for every z
+            g_s[idx] = expf(neg_rate * sp);
+        }
+#pragma unroll
+        for (int r = 0; r < RV; r++)
+            if (tid + r * SCAN_THREADS < TOK * PT) v_s[tid + r * SCAN_THREADS] = g_.v[r];
+        if (tid < TOK) b_s[tid] = 1.0f / (1.0f + expf(-g_.b));
+        __syncthreads();
+        // unit vectors: a wave a token, the sums of squares in lane order then across the wave
+        for (int t = wv; t < TOK; t += SCAN_THREADS / WAVE) {
+            float sk = 0.f, sq = 0.f;
+            for (int n = lane; n < NPAD; n += WAVE) {
+                const float kv = k_s[t * NPAD + n], qv = q_s[t * NPAD + n];
+                sk = fmaf(kv, kv, sk);
+                sq = fmaf(qv, qv, sq);
+            }
+            const float ki = 1.0f / sqrtf(wave_sum(sk) + unit_eps), qi = q_scale / sqrtf(wave_sum(sq) + unit_eps);
+            for (int n = lane; n < NPAD; n += WAVE) {
+                k_s[t * NPAD + n] *= ki;
+                q_s[t * NPAD + n] *= qi;
+            }
+        }
+    };
+    auto chunk = [&](Staged& g_, int c0) {
+        const int nt = n_tok - c0 < TOK ? n_tok - c0 : TOK;
+        __syncthreads();                                   // the walk before has read what is overwritten now
+        stash(g_);
+        __syncthreads();
+        fetch(g_, c0 + 2 * TOK);
+        for (int t = 0; t < nt; t++) {
+            const float4* kt = reinterpret_cast<const float4*>(k_s + t * NPAD + ns * NPT);
+            const float4* qt = reinterpret_cast<const float4*>(q_s + t * NPAD + ns * NPT);
+            const float4* gt = reinterpret_cast<const float4*>(g_s + t * NPAD + ns * NPT);
+            float4 kk[NPT / 4], qq[NPT / 4];
+            float d0 = 0.f, d1 = 0.f;
+#pragma unroll
+            for (int i = 0; i < NPT / 4; i++) {
+                const float4 gg = gt[i];
+                kk[i] = kt[i];
+                qq[i] = qt[i];
+                st[4 * i] *= gg.x;
+                st[4 * i + 1] *= gg.y;
+                st[4 * i + 2] *= gg.z;
+                st[4 * i + 3] *= gg.w;
+                d0 = fmaf(st[4 * i], kk[i].x, d0);
+                d1 = fmaf(st[4 * i + 1], kk[i].y, d1);
+                d0 = fmaf(st[4 * i + 2], kk[i].z, d0);
+                d1 = fmaf(st[4 * i + 3], kk[i].w, d1);
+            }
+            float dot = d0 + d1;
+#pragma unroll
+            for (int off = 1; off < NS; off <<= 1) dot += __shfl_xor(dot, off, WAVE);
+            const float u = b_s[t] * (v_s[t * PT + pl] - dot);
+            float acc0 = 0.f, acc1 = 0.f;
+#pragma unroll
+            for (int i = 0; i < NPT / 4; i++) {
+                st[4 * i] = fmaf(kk[i].x, u, st[4 * i]);
+                st[4 * i + 1] = fmaf(kk[i].y, u, st[4 * i + 1]);
+                st[4 * i + 2] = fmaf(kk[i].z, u, st[4 * i + 2]);
+                st[4 * i + 3] = fmaf(kk[i].w, u, st[4 * i + 3]);
+                acc0 = fmaf(st[4 * i], qq[i].x, acc0);
+                acc1 = fmaf(st[4 * i + 1], qq[i].y, acc1);
+                acc0 = fmaf(st[4 * i + 2], qq[i].z, acc0);
+                acc1 = fmaf(st[4 * i + 3], qq[i].w, acc1);
+            }
+            part_s[t * SCAN_THREADS + tid] = acc0 + acc1;
+        }
+        __syncthreads();
+        for (int idx = tid; idx < nt * PT; idx += SCAN_THREADS) {
+            const int t = idx / PT, pp = idx % PT;
+            if (pz * PT + pp >= P) continue;
+            const float4* sh = reinterpret_cast<const float4*>(part_s + t * SCAN_THREADS + pp * NS);
+            float acc = 0.f;
+#pragma unroll
+            for (int i = 0; i < NS / 4; i++) {
+                const float4 w4 = sh[i];
+                acc = ((acc + w4.x) + w4.y) + w4.z + w4.w;
+            }
+            y[(size_t)(q0 + c0 + t) * ldy + h * P + pz * PT + pp] = acc;
         }
     };
     fetch(set_a, 0);
@@ -263,44 +511,33 @@ __global__ __launch_bounds__(SCAN_THREADS) void linear_scan_kernel(
     for (int i = 0; i < NPT; i++) S[(size_t)i * p_pad * NS] = st[i];
 }
 
-extern "C" int hfa_linear_scan(const void* q, int ldq, const void* k, int ldk, int qk_heads, int qk_dim, const void* v,
-                               int ldv, int n_heads, int v_dim, int dtype, int gate, const float* decay, const void* step,
-                               int step_dtype, int ld_step, const float* step_bias, const float* a_log, const float* skip,
-                               float* state, size_t state_ld, const int* q_start, const int* seq_slot, int n_seqs, float* y,
-                               int ldy, hipStream_t stream) {
-    HFA_REQUIRE(q && k && v && state && q_start && seq_slot && y && n_seqs > 0, "linear_scan: a null argument");
+extern "C" int hfa_delta_scan(const float* q, int ldq, const float* k, int ldk, int qk_heads, int qk_dim, const float* v, int ldv,
+                              int n_heads, int v_dim, const float* a, int lda, const float* dt_bias, const float* a_log,
+                              const float* b, int ldb, float q_scale, float unit_eps, float* state, size_t state_ld,
+                              const int* q_start, const int* seq_slot, int n_seqs, float* y, int ldy, hipStream_t stream) {
+    HFA_REQUIRE(q && k && v && a && dt_bias && a_log && b && state && q_start && seq_slot && y && n_seqs > 0, "delta_scan: a null argument");
     HFA_REQUIRE(n_heads > 0 && qk_heads > 0 && n_heads % qk_heads == 0 && qk_dim > 0 && v_dim > 0,
-                "linear_scan: %d heads over %d heads of keys", n_heads, qk_heads);
-    HFA_REQUIRE(qk_dim <= 256, "linear_scan: a state of %d rows a head is too large (at most 256)", qk_dim);
+                "delta_scan: %d heads over %d heads of keys", n_heads, qk_heads);
+    HFA_REQUIRE(qk_dim <= 256, "delta_scan: a state of %d rows a head is too large (at most 256)", qk_dim);
     HFA_REQUIRE(ldq >= qk_heads * qk_dim && ldk >= qk_heads * qk_dim && ldv >= n_heads * v_dim && ldy >= n_heads * v_dim &&
-                    state_ld >= hfa_linear_scan_state_floats(n_heads, qk_dim, v_dim),
-                "linear_scan: a row is shorter than its heads (a state row holds hfa_linear_scan_state_floats values)");
-    HFA_REQUIRE(dtype == HFA_F32 || dtype == HFA_BF16, "linear_scan: unknown dtype %d", dtype);
-    HFA_REQUIRE((gate == 0 && decay) || (gate == 1 && step && step_bias && a_log && ld_step >= n_heads &&
-                                         (step_dtype == HFA_F32 || step_dtype == HFA_BF16)),
-                "linear_scan: gate 0 needs a decay per head, gate 1 step sizes, their bias and the logarithm of the rate");
+                    lda >= n_heads * qk_dim && ldb >= n_heads && state_ld >= hfa_linear_scan_state_floats(n_heads, qk_dim, v_dim),
+                "delta_scan: a row is shorter than its heads (a state row holds hfa_linear_scan_state_floats values)");
     int ns, npt;
     scan_shape(qk_dim, &ns, &npt);
     const int pt = SCAN_THREADS / ns, p_tiles = (v_dim + pt - 1) / pt;
-    HFA_REQUIRE(n_heads <= 65535 && n_seqs <= 65535 && p_tiles <= 65535, "linear_scan: the step exceeds the grid");
+    HFA_REQUIRE(n_heads <= 65535 && n_seqs <= 65535 && p_tiles <= 65535, "delta_scan: the step exceeds the grid");
     dim3 grid(n_heads, n_seqs, p_tiles);
-#define SCAN_GO(T, TS, NS, NPT)                                                                                          \
-    linear_scan_kernel<T, TS, NS, NPT><<<grid, SCAN_THREADS, 0, stream>>>(                                               \
-        (const T*)q, ldq, (const T*)k, ldk, n_heads / qk_heads, qk_dim, (const T*)v, ldv, v_dim, gate, decay, (const TS*)step, \
-        ld_step, step_bias, a_log, skip, state, state_ld, q_start, seq_slot, y, ldy)
-#define SCAN_SIZES(T, TS)                                          \
-    do {                                                           \
-        if (ns == 4) SCAN_GO(T, TS, 4, 4);                         \
-        else if (ns == 8 && npt == 4) SCAN_GO(T, TS, 8, 4);        \
-        else if (ns == 8) SCAN_GO(T, TS, 8, 8);                    \
-        else if (npt == 4) SCAN_GO(T, TS, 16, 4);                  \
-        else if (npt == 8) SCAN_GO(T, TS, 16, 8);                  \
-        else SCAN_GO(T, TS, 16, 16);                               \
-    } while (0)
-    if (dtype == HFA_F32) { if (step_dtype == HFA_BF16 && gate == 1) SCAN_SIZES(float, bf16); else SCAN_SIZES(float, float); }
-    else { if (step_dtype == HFA_F32 && gate == 1) SCAN_SIZES(bf16, float); else SCAN_SIZES(bf16, bf16); }
-#undef SCAN_SIZES
-#undef SCAN_GO
-    HFA_LAUNCH_CHECK("linear_scan");
+#define DELTA_GO(NS, NPT)                                                                                                       \
+    delta_scan_kernel<NS, NPT><<<grid, SCAN_THREADS, 0, stream>>>(q, ldq, k, ldk, n_heads / qk_heads, qk_dim, v, ldv, v_dim, a, lda, \
+                                                                  dt_bias, a_log, b, ldb, q_scale, unit_eps, state, state_ld,     \
+                                                                  q_start, seq_slot, y, ldy)
+    if (ns == 4) DELTA_GO(4, 4);
+    else if (ns == 8 && npt == 4) DELTA_GO(8, 4);
+    else if (ns == 8) DELTA_GO(8, 8);
+    else if (npt == 4) DELTA_GO(16, 4);
+    else if (npt == 8) DELTA_GO(16, 8);
+    else DELTA_GO(16, 16);
+#undef DELTA_GO
+    HFA_LAUNCH_CHECK("delta_scan");
     return 0;
 }

@@ -21,11 +21,18 @@ _SIGNATURES = {
     "hfa_gemm_rows": [I, P, I, P, I, I, I, I, P, P, I, F, F, P, I, I, I, P, I, P, P, P, I, P, I, P],
     "hfa_gemm_rows_supports": [I, I, I, I, I, I],
     "hfa_rope_store": [P, I, I, P, P, I, I, I, I, I, P, P, P, I, I, P, I, P, P],
-    "hfa_paged_attention": [P, I, I, P, P, I, I, P, I, P, P, P, I, I, I, P, I, I, I, I, I, I, I, I, I, F, P, I, P, c_size_t, I, P],
-    "hfa_group_rmsnorm": [P, I, I, P, P, I, I, P, I, I, I, F, P, I, I, I, P],
+    "hfa_paged_attention": [P, I, I, P, P, I, I, P, I, P, P, P, I, I, I, P, I, I, I, I, I, I, I, I, I, F, P, I, I, P, c_size_t, I, P],
+    "hfa_group_rmsnorm": [P, I, I, P, P, I, I, P, I, I, I, F, P, I, I, I, P, P],
+    "hfa_delta_scan": [P, I, P, I, I, I, P, I, I, I, P, I, P, P, P, I, F, F, P, c_size_t, P, P, I, P, I, P],
+    "hfa_embed_pos": [P, I, P, P, P, P, I, I, I, F, P],
+    "hfa_rmsnorm_add": [P, I, P, I, I, P, P, P, I, I, I, F, F, I, P],
+    "hfa_polynorm": [P, I, I, P, P, I, I, I, I, F, P],
+    "hfa_scale_rows": [P, I, I, I, F, P],
+    "hfa_head_norm_store": [P, I, I, I, I, I, I, P, P, F, P, I, P, P, I, P, I, I, P],
+    "hfa_talk_mix": [P, I, P, P, I, I, P, I, I, I, I, I, I, P],
     "hfa_qkv_prepare": [P, I, I, P, P, I, I, I, I, I, I, P, P, F, P, P, P, P, P, P, I, I, P],
     "hfa_causal_conv": [P, I, I, P, P, I, I, P, c_size_t, P, P, I, I, P, I, I, P],
-    "hfa_linear_scan": [P, I, P, I, I, I, P, I, I, I, I, I, P, P, I, I, P, P, P, P, c_size_t, P, P, I, P, I, P],
+    "hfa_linear_scan": [P, I, P, I, I, I, P, I, I, I, I, I, P, P, I, I, P, P, P, P, c_size_t, P, P, I, P, I, P, P, F, F, P, P],
     "hfa_moe_gated_act": [P, I, P, P, P, I, I, I, I, F, F, F, I, P],
     "hfa_rope_table": [P, P, I, P, I, P],
     "hfa_decode_attention_supports": [I, I, I, I, I, I, I, I],
@@ -74,6 +81,8 @@ def library():
             lib.hfa_attention_prompt_rows.argtypes = []
             lib.hfa_linear_scan_state_floats.restype = c_size_t
             lib.hfa_linear_scan_state_floats.argtypes = [c_int] * 3
+            lib.hfa_linear_scan_max_floats.restype = c_size_t
+            lib.hfa_linear_scan_max_floats.argtypes = [c_int] * 3
             lib.hfa_moe_tile_rows.restype = c_int
             lib.hfa_moe_tile_rows.argtypes = [c_int] * 6
             for name, args in _SIGNATURES.items():

@@ -246,15 +246,111 @@ class Ops:
         return view
 
     # ---- kernels -----------------------------------------------------------
-    def embed(self, table, tokens, out_x):
+    def embed(self, table, tokens, out_x, scale=None, positions=None, inv_freq=None):
+        """``out_x[t] = table[tokens[t]]``; with ``scale`` the row is multiplied by it, and with ``positions`` and
+        ``inv_freq`` (fp32, one per pair of columns) a sinusoidal vector is added: column 2i gets ``sin(p inv_freq[i])``,
+        column 2i + 1 the cosine."""
         self.settle()
         self._source_changes(out_x)
         T = out_x.shape[0]
         if out_x.dtype != torch.float32 or not out_x.is_contiguous() or not table.is_contiguous() \
                 or table.shape[1] != out_x.shape[1]:
             fail(EINVAL, "embed: the output must be contiguous fp32 with the table's width")
-        self._check(self.lib.hfa_embed(table.data_ptr(), _code(table), _ints(tokens, "embed tokens", T),
-                                       out_x.data_ptr(), T, table.shape[1], table.shape[0], self._stream()))
+        if scale is None and positions is None:
+            self._check(self.lib.hfa_embed(table.data_ptr(), _code(table), _ints(tokens, "embed tokens", T),
+                                           out_x.data_ptr(), T, table.shape[1], table.shape[0], self._stream()))
+            return
+        if positions is not None and (inv_freq is None or inv_freq.dtype != torch.float32 or not inv_freq.is_contiguous()
+                                      or inv_freq.numel() < (table.shape[1] + 1) // 2):
+            fail(EINVAL, "embed: a position vector needs one fp32 frequency for every pair of columns")
+        self._check(self.lib.hfa_embed_pos(table.data_ptr(), _code(table), _ints(tokens, "embed tokens", T),
+                                           None if positions is None else _ints(positions, "positions", T),
+                                           None if positions is None else inv_freq.data_ptr(), out_x.data_ptr(), T, table.shape[1],
+                                           table.shape[0], 1.0 if scale is None else float(scale), self._stream()))
+
+    def rmsnorm_add(self, y, weight, eps, out, gate=None, gate_bias=None, scale=1.0, accumulate=True):
+        """``out (+)= scale * rmsnorm(y * sigmoid(gate + gate_bias)) * weight``, all in fp32 (``gate`` None: ``y`` as it is;
+        ``accumulate`` False: ``out`` is overwritten): the norm of a branch's result on its way into the stream."""
+        self.settle()
+        self._source_changes(out)
+        self._scaled.pop(out.data_ptr(), None)
+        R, E = y.shape
+        if y.dtype != torch.float32 or out.dtype != torch.float32 or tuple(out.shape) != (R, E) or weight.dtype != torch.float32 \
+                or weight.numel() != E or not weight.is_contiguous():
+            fail(EINVAL, "rmsnorm_add: y, out and weight must be fp32 and of one width")
+        if gate is not None and (tuple(gate.shape) != (R, E) or (gate_bias is not None and (gate_bias.dtype != torch.float32
+                                                                                            or gate_bias.numel() != E))):
+            fail(EINVAL, "rmsnorm_add: the gate has y's shape, its bias one fp32 value a column")
+        if gate is None and gate_bias is not None:
+            fail(EINVAL, "rmsnorm_add: a gate's bias without the gate")
+        if gate is not None:
+            self._whole(gate)
+        self._check(self.lib.hfa_rmsnorm_add(
+            y.data_ptr(), _rows(y, "norm in"), None if gate is None else gate.data_ptr(), 0 if gate is None else _code(gate),
+            0 if gate is None else _rows(gate, "norm gate"), None if gate_bias is None else gate_bias.data_ptr(), weight.data_ptr(),
+            out.data_ptr(), _rows(out, "norm out"), R, E, float(eps), float(scale), 1 if accumulate else 0, self._stream()))
+
+    def polynorm(self, z, coef, eps, out):
+        """``out = a N(z) + b N(z^2) + c N(z^3) + e`` row by row, ``N(u) = u / sqrt(mean(u^2) + eps)``, ``coef`` = (a, b, c, e)
+        as four fp32 values on the device; sums and powers in fp32."""
+        self.settle()
+        self._whole(z)
+        self._scaled.pop(out.data_ptr(), None)
+        if z.shape != out.shape or z.dim() != 2 or coef.dtype != torch.float32 or coef.numel() != 4 or not coef.is_contiguous():
+            fail(EINVAL, "polynorm: input and output of one shape, four fp32 coefficients")
+        self._check(self.lib.hfa_polynorm(z.data_ptr(), _code(z), _rows(z, "polynorm in"), coef.data_ptr(), out.data_ptr(), _code(out),
+                                          _rows(out, "polynorm out"), z.shape[0], z.shape[1], float(eps), self._stream()))
+
+    def scale_rows(self, x, s):
+        """``x *= s`` on fp32 rows, in place."""
+        self.settle(x)
+        if x.dtype != torch.float32 or x.dim() != 2:
+            fail(EINVAL, "scale_rows: expected an fp32 matrix")
+        if x.shape[0]:
+            self._check(self.lib.hfa_scale_rows(x.data_ptr(), _rows(x, "scale_rows"), x.shape[0], x.shape[1], float(s), self._stream()))
+
+    def head_norm_store(self, qkv, n_heads, n_kv_heads, head_dim, v_head_dim, q_weight, k_weight, eps, q_out, cache, slot_map):
+        """Rows ``[q | k | v]`` (fp32 or bf16): every q head and every k head is RMS-normed over its ``head_dim`` values with a
+        weight of that size which all heads share (None: the part stays as it is); q goes to ``q_out`` ([T, heads * head_dim],
+        the cache's dtype), k and v to ``cache`` at the rows ``slot_map`` names (values transposed inside their page)."""
+        self.settle()
+        self._whole(qkv)
+        self._scaled.pop(q_out.data_ptr(), None)
+        T = qkv.shape[0]
+        QD, KD, VD = n_heads * head_dim, n_kv_heads * head_dim, n_kv_heads * v_head_dim
+        for w, what in ((q_weight, "q"), (k_weight, "k")):
+            if w is not None and (w.dtype != torch.float32 or w.numel() != head_dim or not w.is_contiguous()):
+                fail(EINVAL, f"head_norm_store: the {what} weight must be {head_dim} contiguous fp32 values")
+        if qkv.shape[1] < QD + KD + VD or tuple(q_out.shape) != (T, QD) or q_out.dtype != cache.k.dtype:
+            fail(EINVAL, "head_norm_store: rows of q, k and v in; queries of the cache's dtype out")
+        for c, width in ((cache.k, KD), (cache.v, VD)):
+            if c.dim() != 2 or c.shape[1] != width or not c.is_contiguous():
+                fail(EINVAL, f"head_norm_store: the cache must have one row of {width} values per token")
+        self._check(self.lib.hfa_head_norm_store(
+            qkv.data_ptr(), _code(qkv), _rows(qkv, "qkv"), n_heads, n_kv_heads, head_dim, v_head_dim,
+            None if q_weight is None else q_weight.data_ptr(), None if k_weight is None else k_weight.data_ptr(), float(eps),
+            q_out.data_ptr(), _rows(q_out, "queries"), cache.k.data_ptr(), cache.v.data_ptr(), _code(cache.k),
+            _ints(slot_map, "slot_map", T), cache.page_tokens, T, self._stream()))
+
+    def talk_mix(self, cross, talk, n_heads, n_kv_heads, v_head_dim, out, gate=None):
+        """``out[t, h] = sigmoid(gate[t, h]) * sum_g talk[h, g] A[t, g, group of h]``: the heads' attention weights mixed after
+        the softmax, as the same mix of what each head's weights give on the values of h's group. ``cross`` is
+        ``paged_attention(..., cross_values=True)``'s output, ``talk`` fp32 [heads, heads]; ``gate`` None: no gate."""
+        self.settle()
+        self._scaled.pop(out.data_ptr(), None)
+        T = out.shape[0]
+        OD = n_heads * v_head_dim
+        if tuple(cross.shape) != (T, n_kv_heads * OD) or not cross.is_contiguous() or out.shape[1] != OD \
+                or talk.dtype != torch.float32 or tuple(talk.shape) != (n_heads, n_heads) or not talk.is_contiguous():
+            fail(EINVAL, "talk_mix: cross [T, groups * heads * v_head_dim], talk fp32 [heads, heads], out [T, heads * v_head_dim]")
+        if gate is not None:
+            self._whole(gate)
+            if gate.shape[0] != T or gate.shape[1] != OD:
+                fail(EINVAL, "talk_mix: the gate has the output's shape")
+        self._check(self.lib.hfa_talk_mix(cross.data_ptr(), _code(cross), talk.data_ptr(), None if gate is None else gate.data_ptr(),
+                                          0 if gate is None else _code(gate), 0 if gate is None else _rows(gate, "gate"),
+                                          out.data_ptr(), _code(out), _rows(out, "talk_mix out"), T, n_heads, n_kv_heads, v_head_dim,
+                                          self._stream()))
 
     def rmsnorm(self, x, weight, eps, out, rows=None, lazy=False):
         """``out[r] = norm(x[rows[r]])``. ``lazy``: the caller promises that ``out`` is read by ``gemm`` alone. Then,
@@ -525,18 +621,22 @@ class Ops:
             None if pend is None or pend.bias is None else pend.bias.data_ptr(), self._stream()))
 
     def paged_attention(self, q, n_heads, n_kv_heads, head_dim, cache, step, window, scale, out, slopes=None,
-                        v_head_dim=None, mask_chunk=0, sink=False):
+                        v_head_dim=None, mask_chunk=0, sink=False, cross_values=False):
         """Attention of the first ``n_heads * head_dim`` columns of ``q`` over ``cache``. ``slopes``
         (fp32, one per query head): the score of key j for the query at p gets ``slopes[h] * (j - p)``
         added, for position encodings that enter the scores; the plain kernel then runs, as it does when
         value heads have a size of their own (``v_head_dim``; ``out`` then has that many columns a head).
         ``mask_chunk`` > 0: a query sees only the keys of its own run of that many positions, counted from 0.
-        ``sink``: the softmax's denominator holds one more term of score 0 that has no value."""
+        ``sink``: the softmax's denominator holds one more term of score 0 that has no value. ``cross_values``: every
+        head's weights are applied to the values of every key/value group; ``out`` is ``[T, groups * heads * v_head_dim]``,
+        round r of head h (at ``(r * heads + h) * v_head_dim``) being its weights on the values of group (h's group + r) mod
+        groups (see ``talk_mix``)."""
         v_head_dim = head_dim if v_head_dim is None else int(v_head_dim)
         mask_chunk = int(mask_chunk)
         self._scaled.pop(out.data_ptr(), None)               # whatever `out` held, it is no norm's lazy output any more
         lr = self._lazy_rope
         if lr is not None and lr.qkv.data_ptr() == q.data_ptr() and lr.cache is cache and slopes is None and not sink \
+                and not cross_values \
                 and step.max_q_len == 1 and step.n_seqs == q.shape[0] and not self.force_plain_attention \
                 and out.dtype == torch.bfloat16 and v_head_dim == head_dim and lr.args[4] == n_heads and lr.args[6] == head_dim \
                 and lr.args[5] in (0, n_kv_heads) and cache.k.shape[1] == n_kv_heads * head_dim \
@@ -558,7 +658,9 @@ class Ops:
         _ints(step.q_start, "q_start", step.n_seqs + 1)
         # the matrix-core kernels address the cache with 32-bit element offsets and 24-bit row numbers
         too_large = cache.k.numel() >= 1 << 32 or cache.k.shape[0] >= 1 << 24
-        plain = self.force_plain_attention or slopes is not None or too_large
+        plain = self.force_plain_attention or slopes is not None or too_large or bool(cross_values)
+        if cross_values and out.shape[1] != n_kv_heads * n_heads * v_head_dim:
+            fail(EINVAL, "paged_attention: with cross_values the output holds groups * heads * v_head_dim columns")
         if too_large and q.dtype == torch.bfloat16 and not self._said_cache_too_large:
             self._said_cache_too_large = True        # right, but many times slower: say so once
             print(f"[hf_cpu_amd] a layer's cache of {cache.k.shape[0]} rows x {cache.k.shape[1]} is beyond what the "
@@ -572,7 +674,7 @@ class Ops:
                 step.token_slot.data_ptr() + 4 * first, step.positions.data_ptr() + 4 * first, q_start.data_ptr(), n_seqs,
                 max_q_len, step.max_seq_len, out.data_ptr() + first * ldo * out.element_size(), ldo, n_tokens, n_heads,
                 n_kv_heads, head_dim, v_head_dim, cache.page_tokens, int(window), mask_chunk, float(scale),
-                None if slopes is None else slopes.data_ptr(), 1 if sink else 0, self.attn_workspace.data_ptr(),
+                None if slopes is None else slopes.data_ptr(), 1 if sink else 0, 1 if cross_values else 0, self.attn_workspace.data_ptr(),
                 self.attn_workspace.numel(), 1 if plain else 0, self._stream()))
 
         # Decoded tokens beside prompt portions: one call would send all of them to the kernel for prompt
@@ -627,11 +729,12 @@ class Ops:
     # ---- norms in groups, queries and keys normed whole, mixers with per-request state -------------------------------
     GATES = {None: 0, "silu_before": 1, "sigmoid_after": 2}
 
-    def group_rmsnorm(self, x, weight, eps, groups, out, rows=None, gate=None, gate_kind=None):
+    def group_rmsnorm(self, x, weight, eps, groups, out, rows=None, gate=None, gate_kind=None, row_scale=None):
         """``out[r] = norm(x[rows[r]])``: the row is cut into ``groups`` equal runs, each divided by its own root mean
         square (``eps`` inside the root), the whole times ``weight``; sums in fp32. ``gate`` (a matrix with the rows of
         ``out``) with ``gate_kind`` ``silu_before`` (the row times silu(gate) is normed) or ``sigmoid_after`` (the normed
-        row is multiplied by sigmoid(gate))."""
+        row is multiplied by sigmoid(gate)). ``row_scale`` (fp32 [rows, groups]): run g of row r is multiplied by
+        ``row_scale[r, g]`` before everything else (a recurrence's denominator, a head at a time)."""
         self.settle()
         self._whole(x)
         self._scaled.pop(out.data_ptr(), None)
@@ -644,11 +747,15 @@ class Ops:
             fail(EINVAL, "group_rmsnorm: without row indices the output must have x's rows")
         if gate is not None and (gate.shape[0] != R or gate.shape[1] != E or rows is not None):
             fail(EINVAL, "group_rmsnorm: the gate has the output's shape, and no rows are gathered with it")
+        if row_scale is not None and (rows is not None or row_scale.dtype != torch.float32 or not row_scale.is_contiguous()
+                                      or tuple(row_scale.shape) != (R, int(groups))):
+            fail(EINVAL, "group_rmsnorm: row_scale is fp32 [rows, groups], and no rows are gathered with it")
         self._check(self.lib.hfa_group_rmsnorm(
             x.data_ptr(), _code(x), _rows(x, "norm in"), weight.data_ptr(), out.data_ptr(), _code(out), _rows(out, "norm out"),
             None if rows is None else _ints(rows, "norm rows", R), R, E, int(groups), float(eps),
             None if gate is None else gate.data_ptr(), 0 if gate is None else _code(gate),
-            0 if gate is None else _rows(gate, "norm gate"), self.GATES[gate_kind], self._stream()))
+            0 if gate is None else _rows(gate, "norm gate"), self.GATES[gate_kind],
+            None if row_scale is None else row_scale.data_ptr(), self._stream()))
 
     PAIRINGS = {"split_half": 0, "interleaved": 1}
 
@@ -712,36 +819,57 @@ class Ops:
             self.ACTIVATIONS["silu"] if activation else 0, self._stream()))
 
     @staticmethod
-    def scan_state_floats(n_heads, qk_dim, v_dim):
+    def scan_state_floats(n_heads, qk_dim, v_dim, normalizer=False):
         """The fp32 values of a request's state row that ``linear_scan`` needs for ``n_heads`` states of ``qk_dim`` x ``v_dim``:
         the kernel keeps them in the order its lanes read them, both sizes padded to what a block walks (the library's
-        ``hfa_linear_scan_state_floats``, mirrored here so that a cache can be planned without the library)."""
+        ``hfa_linear_scan_state_floats``, mirrored here so that a cache can be planned without the library). ``normalizer``
+        (exponential gates): one more column a head, and the running maximum once for every block of columns."""
         lanes = 16 if qk_dim >= 64 else 8 if qk_dim > 16 else 4
         per = -(-qk_dim // lanes)
         per = 4 if per <= 4 else 8 if per <= 8 else 16
         columns = 256 // lanes
+        if normalizer:
+            blocks = -(-(v_dim + 1) // columns)
+            return n_heads * lanes * per * blocks * columns + n_heads * blocks
         return n_heads * lanes * per * (-(-v_dim // columns) * columns)
 
     def linear_scan(self, q, k, v, qk_heads, qk_dim, n_heads, v_dim, state, step, y, decay=None, step_size=None,
-                    step_bias=None, a_log=None, skip=None):
+                    step_bias=None, a_log=None, skip=None, exp_gates=None, q_scale=1.0, denom=None):
         """The recurrence over a matrix state per head, along each request's tokens from its row of ``state`` ([slots, >=
         ``scan_state_floats``] fp32, in the kernel's own order, left there for the next step): ``S <- a_t S + k_t (b_t v_t)^T``, ``y_t = S^T q_t +
         skip[h] v_t`` (fp32). Head h reads queries and keys of head ``h // (n_heads / qk_heads)``. With ``decay`` (fp32, one
         per head): ``a_t = decay[h]``, ``b_t = 1``. With ``step_size`` ([T, heads]), ``step_bias`` and ``a_log`` (fp32 per head):
-        ``dt = softplus(step_size + step_bias)``, ``a_t = exp(-exp(a_log) dt)``, ``b_t = dt``."""
+        ``dt = softplus(step_size + step_bias)``, ``a_t = exp(-exp(a_log) dt)``, ``b_t = dt``. With ``exp_gates`` = (i [T, heads],
+        f [T, heads], i_bias, f_bias (fp32 per head), cap): exponential input gates and sigmoid forget gates, both soft-capped,
+        under a running maximum m that is kept beside the states (``scan_state_floats(..., normalizer=True)``):
+        ``li = cap tanh((i + i_bias) / cap)``, ``lf = logsigmoid(cap tanh((f + f_bias) / cap))``, ``m_t = max(lf + m, li)``,
+        ``a_t = exp(lf + m - m_t)``, ``b_t = exp(li - m_t)``; the state carries ``n_t = a_t n + b_t k_t`` as one more column and
+        ``denom`` (fp32 [T, heads]) receives ``1 / (max(|n_t . q_t|, exp(-m_t)) + 1e-6)``, by which the reader multiplies
+        ``y``. ``q_scale`` multiplies the queries."""
         self.settle()
         for t in (q, k, v):
             self._whole(t)
         T = y.shape[0]
-        gate = 0 if decay is not None else 1
+        gate = 0 if decay is not None else 2 if exp_gates is not None else 1
+        gi = gf = gib = gfb = None
+        cap = 0.0
+        if gate == 2:
+            gi, gf, gib, gfb, cap = exp_gates
+            step_size, step_bias = gi, gib
+            if gf.dtype != gi.dtype or gf.shape != gi.shape or _rows(gf, "scan f") != _rows(gi, "scan i") or gfb.dtype != torch.float32 \
+                    or gfb.numel() != n_heads or denom is None or denom.dtype != torch.float32 or tuple(denom.shape) != (T, n_heads) \
+                    or not denom.is_contiguous() or skip is not None or not cap > 0.0:
+                fail(EINVAL, "linear_scan: exponential gates are (i, f, i_bias, f_bias, cap > 0) with i and f alike, and denom fp32 [T, heads]")
         if q.dtype != k.dtype or q.dtype != v.dtype or y.dtype != torch.float32 or state.dtype != torch.float32 \
                 or state.stride(1) != 1 or q.shape[0] != T or k.shape[0] != T or v.shape[0] != T or y.shape[1] != n_heads * v_dim:
             fail(EINVAL, "linear_scan: q, k and v of one dtype and the step's rows, fp32 output and state")
         for t, what in ((decay, "decay"), (step_bias, "step_bias"), (a_log, "a_log"), (skip, "skip")):
             if t is not None and (t.dtype != torch.float32 or t.numel() != n_heads or not t.is_contiguous()):
                 fail(EINVAL, f"linear_scan: {what} must be one fp32 value a head")
-        if state.shape[1] < self.scan_state_floats(n_heads, qk_dim, v_dim) or qk_dim > 256:
+        if state.shape[1] < self.scan_state_floats(n_heads, qk_dim, v_dim, normalizer=gate == 2) or qk_dim > 256:
             fail(EINVAL, f"linear_scan: a state row of {state.shape[1]} values for {n_heads} states of {qk_dim} x {v_dim} (at most 256 rows)")
+        if gate == 2 and step_size.shape[0] != T:
+            fail(EINVAL, "linear_scan: the gates' inputs have the step's rows")
         if gate == 1 and (step_size is None or step_bias is None or a_log is None or step_size.shape[0] != T):
             fail(EINVAL, "linear_scan: without a fixed decay give step_size, step_bias and a_log")
 
@@ -752,7 +880,31 @@ class Ops:
             n_heads, v_dim, _code(q), gate, ptr(decay), ptr(step_size), 0 if step_size is None else _code(step_size),
             0 if step_size is None else _rows(step_size, "scan step"), ptr(step_bias), ptr(a_log), ptr(skip), state.data_ptr(),
             state.stride(0), _ints(step.q_start, "q_start", step.n_seqs + 1), _ints(step.seq_slot, "seq_slot", step.n_seqs),
-            step.n_seqs, y.data_ptr(), _rows(y, "scan out"), self._stream()))
+            step.n_seqs, y.data_ptr(), _rows(y, "scan out"), ptr(gf), ptr(gfb), float(cap), float(q_scale), ptr(denom), self._stream()))
+
+    def delta_scan(self, q, k, v, qk_heads, qk_dim, n_heads, v_dim, a, dt_bias, a_log, b, state, step, y, q_scale=1.0, unit_eps=1e-6):
+        """The gated delta rule over a matrix state per head, along each request's tokens from its row of ``state`` (fp32,
+        ``scan_state_floats`` values in ``linear_scan``'s order): ``g_t = exp(-exp(a_log[h]) softplus(a[t, h] + dt_bias[h]))``, one
+        decay per key channel (``a`` [T, heads * qk_dim], ``dt_bias`` [heads * qk_dim]); ``S <- g_t * S`` row by row;
+        ``u = sigmoid(b[t, h]) (v_t - S^T k_t)``; ``S <- S + k_t u^T``; ``y_t = S^T q_t``. ``q_t`` and ``k_t`` are first divided
+        by ``sqrt(sum of squares + unit_eps)`` and ``q_t`` multiplied by ``q_scale``. Head h reads queries and keys of head
+        ``h // (n_heads / qk_heads)``. Every input is fp32, as is every operation."""
+        self.settle()
+        T = y.shape[0]
+        for t, what in ((q, "q"), (k, "k"), (v, "v"), (a, "a"), (b, "b"), (y, "y"), (state, "state")):
+            if t.dtype != torch.float32 or t.dim() != 2 or t.stride(1) != 1 or (what != "state" and t.shape[0] != T):
+                fail(EINVAL, f"delta_scan: {what} must be an fp32 matrix with the step's rows")
+        if dt_bias.dtype != torch.float32 or dt_bias.numel() != n_heads * qk_dim or not dt_bias.is_contiguous() \
+                or a_log.dtype != torch.float32 or a_log.numel() != n_heads or not a_log.is_contiguous():
+            fail(EINVAL, "delta_scan: dt_bias is one fp32 value a (head, key channel), a_log one a head")
+        if state.shape[1] < self.scan_state_floats(n_heads, qk_dim, v_dim) or qk_dim > 256 or y.shape[1] != n_heads * v_dim \
+                or a.shape[1] < n_heads * qk_dim or b.shape[1] < n_heads:
+            fail(EINVAL, f"delta_scan: a state row of {state.shape[1]} values for {n_heads} states of {qk_dim} x {v_dim} (at most 256 rows)")
+        self._check(self.lib.hfa_delta_scan(
+            q.data_ptr(), _rows(q, "scan q"), k.data_ptr(), _rows(k, "scan k"), qk_heads, qk_dim, v.data_ptr(), _rows(v, "scan v"),
+            n_heads, v_dim, a.data_ptr(), _rows(a, "scan a"), dt_bias.data_ptr(), a_log.data_ptr(), b.data_ptr(), _rows(b, "scan b"),
+            float(q_scale), float(unit_eps), state.data_ptr(), state.stride(0), _ints(step.q_start, "q_start", step.n_seqs + 1),
+            _ints(step.seq_slot, "seq_slot", step.n_seqs), step.n_seqs, y.data_ptr(), _rows(y, "scan out"), self._stream()))
 
     # ---- layer norm, plain activations, soft cap -----------------------------------------------------------------
     def layernorm(self, x, weight, bias, eps, out, rows=None):

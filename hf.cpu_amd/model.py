@@ -26,6 +26,24 @@ def compute_dtype(name):
     return COMPUTE_DTYPES[name]
 
 
+def _number_needs(need, needs):
+    """Gives ``need`` (a PagedKV, a FixedState, None, or a dict of these by name: a part that keeps several caches, or that
+    owns parts which do) its places in the flat list ``needs``; returns the place, or a dict of places in the same shape."""
+    if isinstance(need, dict):
+        return {name: _number_needs(n, needs) for name, n in need.items()}
+    if need is not None and not isinstance(need, (PagedKV, FixedState)):
+        raise TypeError(f"cache_need() returned {need!r}")
+    needs.append(need)
+    return len(needs) - 1
+
+
+def _views_of(slot, caches):
+    """The cache view of a place, or the dict of views of a dict of places."""
+    if isinstance(slot, dict):
+        return {name: _views_of(k, caches) for name, k in slot.items()}
+    return caches[slot]
+
+
 class Layer:
     """A layer's block and the parts it arranges, by the names the plan gave them (also as attributes)."""
 
@@ -127,14 +145,11 @@ class Model:
             slots = {}
             for name, part in self.layers[e.layer].cache_parts():
                 need = part.cache_need() if e.cache_of is None else None
-                if need is not None and not isinstance(need, (PagedKV, FixedState)):
-                    raise TypeError(f"{type(part).__name__}.cache_need() returned {need!r}")
-                slots[name] = len(needs)
-                needs.append(need)
+                slots[name] = _number_needs(need, needs)
                 if e.cache_of is not None and hasattr(part, "reads_cache"):
                     # what the reader sees of the other entry's storage decides with it how long rows are kept
                     k = self.cache_slots[e.cache_of].get(name)
-                    if k is not None and isinstance(needs[k], PagedKV):
+                    if isinstance(k, int) and isinstance(needs[k], PagedKV):
                         needs[k] = part.reads_cache(needs[k])
             self.cache_slots.append(slots)
         return needs
@@ -142,7 +157,8 @@ class Model:
     # ---- the forward pass of one step ----------------------------------------
     def forward(self, ops, step, caches, logits_out):
         """Runs ``step``'s tokens through the schedule. ``caches[k]`` is the cache view
-        of entry ``k`` of ``cache_needs()`` (None if it needs none). Writes fp32 logits for
+        of entry ``k`` of ``cache_needs()`` (None if it needs none); a part whose ``cache_need()`` is a dict of needs by name
+        gets a dict of views by the same names. Writes fp32 logits for
         ``step.logit_rows`` into ``logits_out`` ([R, V]; R may be 0)."""
         with ops.on_current_stream(), ops.section("total"):
             self._forward(ops, step, caches, logits_out)
@@ -156,7 +172,7 @@ class Model:
         for i, e in enumerate(self.schedule):
             layer = self.layers[e.layer]
             own = e.cache_of is None
-            mine = {name: caches[k] for name, k in self.cache_slots[i if own else e.cache_of].items()}
+            mine = {name: _views_of(k, caches) for name, k in self.cache_slots[i if own else e.cache_of].items()}
             layer.block.forward(ops, step, x, layer.named, mine, write_cache=own)
         R = step.n_logit_rows
         if R:

@@ -8,7 +8,7 @@ from .. import memory
 
 from ..registry import make_part, register_part
 from ..status import EINVAL, fail
-from .base import PagedKV, ParamSpec, Part
+from .base import FixedState, PagedKV, ParamSpec, Part
 
 
 @register_part("mixer", "attention")
@@ -37,14 +37,26 @@ class Attention(Part):
     are kept for the step; ``"blend"``: ``v <- (1 - l) v + l v_first`` with the scalar tensor ``v_mix`` (name in
     ``names``) and the kept values of the same token; the blended values are what is cached. A ``"first"`` layer holds the
     scalar too, unused.
+
+    ``conv_taps`` K > 1: q, k and v pass a causal convolution over the last K tokens per channel straight after the
+    projection (tensors ``q_conv``, ``k_conv``, ``v_conv`` in ``names``, [channels, K], the last column the current token's, no
+    bias, zeros before a sequence's start); the last K - 1 projected rows of a request are part of its state, so the mixer
+    then needs ``{"kv": PagedKV, "conv": FixedState}``. ``head_norm`` = eps: queries and keys are RMS-normed head by head over
+    ``head_dim`` with weights of that size which all heads share (``q_norm``, ``k_norm``). ``talk``: the heads' softmax weights
+    are mixed after the softmax, ``weight_h <- sum_g talk[h, g] weight_g`` (tensor ``talk`` [heads, heads]), and head h applies
+    its mixed weights to the values of its own group. ``out_gate``: the concatenated heads are multiplied by
+    ``sigmoid(Wg h)`` (tensor ``g``) before the output projection. Any of these four takes the mixer through a path of its
+    own (``_forward_shaped``), which knows no rotation, no ``own_kv=False`` and none of ``qk_norm``, ``sink``, ``v_mix``.
+    ``forward(..., accumulate=False)`` writes ``x = ...`` instead of adding.
     """
     graph_safe = True
     lazy_input_ok = True
+    can_overwrite = True
 
 
     def __init__(self, hidden_size, n_heads, n_kv_heads, head_dim, qkv_bias, window, position,
                  scale=None, out_bias=False, v_head_dim=None, prefix="", mask_chunk=0, own_kv=True, names=None,
-                 qk_norm=None, sink=False, v_mix=None):
+                 qk_norm=None, sink=False, v_mix=None, conv_taps=0, head_norm=None, talk=False, out_gate=False):
         """``v_head_dim``: the size of a value head where it is not ``head_dim`` (key rows of the cache are
         then ``n_kv_heads * head_dim`` wide, value rows ``n_kv_heads * v_head_dim``, and the output
         projection reads ``n_heads * v_head_dim`` columns; such a mixer runs the plain kernels)."""
@@ -62,8 +74,20 @@ class Attention(Part):
         self.own_kv = bool(own_kv)
         self.names = {n: f"{n}_proj.weight" for n in "qkvo"}
         self.names.update({f"{n}_bias": f"{n}_proj.bias" for n in "qkvo"})
-        self.names.update(q_norm="q_norm.weight", k_norm="k_norm.weight", v_mix="v_mix")
+        self.names.update(q_norm="q_norm.weight", k_norm="k_norm.weight", v_mix="v_mix", talk="talk", g="g_proj.weight",
+                          q_conv="q_conv.weight", k_conv="k_conv.weight", v_conv="v_conv.weight")
         self.names.update(names or {})
+        self.conv_taps = int(conv_taps)
+        self.head_norm = None if head_norm is None else float(head_norm)
+        self.talk, self.out_gate = bool(talk), bool(out_gate)
+        self.shaped = self.conv_taps > 1 or self.head_norm is not None or self.talk or self.out_gate
+        if self.shaped and (position.kind != "none" or not own_kv or qk_norm is not None or sink or v_mix or qkv_bias or window
+                            or mask_chunk):
+            fail(EINVAL, "attention: a convolution, per-head norms, mixed heads and an output gate go without rotation, biases, "
+                         "windows and the other options")
+        if not 0 <= self.conv_taps <= 8:
+            fail(EINVAL, f"attention: a convolution over {self.conv_taps} tokens (at most 8)")
+        self.taps = self.talk_w = None
         self.qk_norm = None if qk_norm is None else float(qk_norm)
         self.sink = bool(sink)
         if v_mix not in (None, "first", "blend") or (v_mix and not own_kv):
@@ -94,6 +118,14 @@ class Attention(Part):
                 specs.append(ParamSpec(p + nm["k_norm"], (self.KD,), "vector", ("one_plus_normal", 0.1)))
         if self.v_mix:
             specs.append(ParamSpec(p + nm["v_mix"], (), "vector", ("normal", 0.3), optional=self.v_mix == "first"))
+        if self.conv_taps > 1:
+            specs += [ParamSpec(p + nm[n + "_conv"], (widths[n], self.conv_taps), "vector", ("normal", 0.3)) for n in "qkv"]
+        if self.head_norm is not None:
+            specs += [ParamSpec(p + nm[n], (self.D,), "vector", ("one_plus_normal", 0.1)) for n in ("q_norm", "k_norm")]
+        if self.talk:
+            specs.append(ParamSpec(p + nm["talk"], (self.H, self.H), "vector", ("normal", 0.3)))
+        if self.out_gate:
+            specs.append(ParamSpec(p + nm["g"], (self.OD, self.E)))
         return specs
 
     def _projections(self):
@@ -103,7 +135,10 @@ class Attention(Part):
         if not self.own_kv:
             fail(EINVAL, f"attention '{self.prefix}' has no keys and values of its own: its schedule entry must read "
                          "another entry's cache")
-        return PagedKV(self.KD, self.VD, self.window, self.mask_chunk)
+        kv = PagedKV(self.KD, self.VD, self.window, self.mask_chunk)
+        if self.conv_taps > 1:
+            return {"kv": kv, "conv": FixedState((self.conv_taps - 1) * (self.QD + self.KD + self.VD))}
+        return kv
 
     def reads_cache(self, need):
         """``need`` of the mixer whose storage this one reads, widened by what this one sees of it."""
@@ -113,6 +148,8 @@ class Attention(Part):
         p, nm = self.prefix, self.names
         # One matrix for the three projections that share an input: rows of q, then k, then v.
         mats = [params[p + nm[n]] for n in self._projections()]
+        if self.out_gate:
+            mats.append(params[p + nm["g"]])             # the gate reads the same input: one product for all four
         dt = torch.float32 if any(m.dtype == torch.float32 for m in mats) else mats[0].dtype
         self.w_qkv = memory.cat([m.to(dt) for m in mats], 0, f"{p}q, k and v in one matrix")
         if self.qkv_bias:
@@ -127,8 +164,50 @@ class Attention(Part):
             self.k_norm_w = params[p + nm["k_norm"]] if self.own_kv else None
         if self.v_mix == "blend":
             self.v_blend = params[p + nm["v_mix"]].reshape(1)
+        if self.conv_taps > 1:
+            self.taps = memory.cat([params[p + nm[n + "_conv"]] for n in "qkv"], 0, f"{p}taps of q, k and v in one matrix").contiguous()
+        if self.head_norm is not None:
+            self.q_norm_w, self.k_norm_w = params[p + nm["q_norm"]].contiguous(), params[p + nm["k_norm"]].contiguous()
+        if self.talk:
+            self.talk_w = params[p + nm["talk"]].contiguous()
+        elif self.out_gate:                              # the gate rides in the kernel that mixes heads: an identity mix
+            self.talk_w = memory.to_device(torch.eye(self.H, dtype=torch.float32), ops.device, f"{p}identity mix of heads")
 
-    def forward(self, ops, step, h, cache, x, write_cache=True):
+    def _forward_shaped(self, ops, step, h, cache, x, accumulate):
+        """The path of a mixer with a convolution, per-head norms, mixed heads or an output gate (see the class)."""
+        T = h.shape[0]
+        C = self.QD + self.KD + self.VD
+        kv = cache["kv"] if isinstance(cache, dict) else cache
+        proj = ops.scratch("qkv", (T, self.w_qkv.shape[0]), ops.act_dtype)
+        with ops.section("qkv"):
+            ops.gemm(h, self.w_qkv, proj)
+        rows = proj[:, :C]
+        with ops.section("qkv_prepare"):
+            if self.conv_taps > 1:
+                rows = ops.scratch("qkv_conv", (T, C), torch.float32)
+                ops.causal_conv(proj[:, :C], self.taps, None, cache["conv"].state, step, rows)
+            q = ops.scratch("q_normed", (T, self.QD), ops.act_dtype)
+            ops.head_norm_store(rows, self.H, self.G, self.D, self.Dv, self.q_norm_w, self.k_norm_w, self.head_norm or 0.0, q, kv,
+                                step.group(kv.group).slot_map)
+        att = ops.scratch("att", (T, self.OD), ops.act_dtype)
+        with ops.section("attn"):
+            if self.talk_w is None:
+                ops.paged_attention(q, self.H, self.G, self.D, kv, step, 0, self.scale, att, v_head_dim=self.Dv)
+            else:
+                cross = ops.scratch("att_cross", (T, self.G * self.OD), ops.act_dtype)
+                ops.paged_attention(q, self.H, self.G, self.D, kv, step, 0, self.scale, cross, v_head_dim=self.Dv, cross_values=True)
+                ops.talk_mix(cross, self.talk_w, self.H, self.G, self.Dv, att, gate=proj[:, C:] if self.out_gate else None)
+        with ops.section("wo"):
+            if accumulate:
+                ops.gemm(att, self.w_o, x, accumulate=True, defer=True)
+            else:
+                ops.gemm(att, self.w_o, x)
+
+    def forward(self, ops, step, h, cache, x, write_cache=True, accumulate=True):
+        if self.shaped:
+            if not write_cache:
+                fail(EINVAL, f"attention '{self.prefix}': this mixer cannot read another entry's cache")
+            return self._forward_shaped(ops, step, h, cache, x, accumulate)
         T = h.shape[0]
         if write_cache and not self.own_kv:
             fail(EINVAL, f"attention '{self.prefix}' has no keys and values to write")
@@ -157,4 +236,7 @@ class Attention(Part):
                                 slopes=getattr(self.position, "score_slopes", None), v_head_dim=self.Dv,
                                 mask_chunk=self.mask_chunk, sink=self.sink)
         with ops.section("wo"):
-            ops.gemm(att, self.w_o, x, bias=self.b_o, accumulate=True, defer=True)
+            if accumulate:
+                ops.gemm(att, self.w_o, x, bias=self.b_o, accumulate=True, defer=True)
+            else:
+                ops.gemm(att, self.w_o, x, bias=self.b_o)

@@ -24,7 +24,8 @@ class ParamSpec:
     """One tensor of the checkpoint. ``kind``: "matrix" (a matrix-product operand,
     held in the compute dtype unless stored in 32-bit), "vector" (widened to fp32),
     "table" (integers, held as int32). ``init`` is the random-weights rule:
-    ("normal", std) or ("one_plus_normal", std)."""
+    ("normal", std) or ("one_plus_normal", std). A 0 in ``shape`` stands for a size that only the checkpoint's tensor
+    gives (random weights cannot be made for such a spec: the part then has to be told the size)."""
     name: str
     shape: tuple
     kind: str = "matrix"

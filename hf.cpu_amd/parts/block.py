@@ -1,6 +1,8 @@
 """Arrangements of a layer's parts around the residual stream."""
+import torch
+
 from ..registry import register_part
-from .base import Part
+from .base import ParamSpec, Part
 
 
 @register_part("block", "prenorm")
@@ -46,6 +48,77 @@ class ParallelBlock(Part):
         ff = parts.get("feed_forward")
         if ff is not None:
             ff.forward(ops, step, h, x)
+
+
+@register_part("block", "sandwich")
+class SandwichBlock(Part):
+    """Norms before and after each sublayer: ``h = norm1(x); x += norm1b(gate(h) * mixer(h))``, then the same with ``norm2``,
+    ``feed_forward`` and ``norm2b`` where the layer has a feed-forward. ``gate(h) = sigmoid(W h + b)`` multiplies the
+    sublayer's result element by element before the second norm; ``gates`` names the tensors of each sublayer's gate after
+    ``prefix``, ``{"mixer": (W, b), "feed_forward": (W, b)}`` (a sublayer that is not named has no gate). The sublayer's
+    result, the gate, the second norm and the sum into the stream are fp32. The norms after the sublayers are parts with an
+    ``add_into`` method (``rmsnorm``)."""
+    graph_safe = True
+
+    def __init__(self, hidden_size, gates=None, prefix=""):
+        super().__init__(prefix)
+        self.E = hidden_size
+        self.gate_names = {k: tuple(v) for k, v in (gates or {}).items()}
+        self.gate_w = {}
+
+    def param_specs(self):
+        specs = []
+        for w, b in self.gate_names.values():
+            specs += [ParamSpec(self.prefix + w, (self.E, self.E)), ParamSpec(self.prefix + b, (self.E,), "vector")]
+        return specs
+
+    def bind(self, params, ops):
+        self.gate_w = {k: (params[self.prefix + w], params[self.prefix + b]) for k, (w, b) in self.gate_names.items()}
+
+    def _sublayer(self, ops, step, x, h, which, part, post, run):
+        """``x += post(gate(h) * part(h))``; ``run(y, overwrite)`` makes the part write (or add) its result into ``y``."""
+        T = x.shape[0]
+        y = ops.scratch("branch", (T, self.E), torch.float32)
+        if getattr(part, "can_overwrite", False):
+            run(y, True)
+        else:                                  # a part that only knows how to add: into zeros
+            ops.settle()
+            y.zero_()
+            run(y, False)
+        gate = bias = None
+        if which in self.gate_w:
+            w, bias = self.gate_w[which]
+            gate = ops.scratch("branch_gate", (T, self.E), torch.float32)
+            with ops.section("gate"):
+                ops.gemm(h, w, gate)
+        with ops.section("post_norm"):
+            post.add_into(ops, y, x, gate=gate, gate_bias=bias)
+
+    def forward(self, ops, step, x, parts, caches, write_cache=True):
+        """``parts``: norm1, mixer, norm1b and, if the layer has a feed-forward, norm2, feed_forward, norm2b."""
+        h = ops.scratch("normed", (x.shape[0], self.E), ops.act_dtype)
+        parts["norm1"].forward(ops, x, h)
+        ops.settle(x)
+        mixer, cache = parts["mixer"], caches.get("mixer")
+
+        def run_mixer(y, overwrite):
+            if overwrite:
+                mixer.forward(ops, step, h, cache, y, write_cache, accumulate=False)
+            else:
+                mixer.forward(ops, step, h, cache, y, write_cache)
+        self._sublayer(ops, step, x, h, "mixer", mixer, parts["norm1b"], run_mixer)
+        ff = parts.get("feed_forward")
+        if ff is None:
+            return
+        parts["norm2"].forward(ops, x, h)
+        ops.settle(x)
+
+        def run_ff(y, overwrite):
+            if overwrite:
+                ff.forward(ops, step, h, y, accumulate=False)
+            else:
+                ff.forward(ops, step, h, y)
+        self._sublayer(ops, step, x, h, "feed_forward", ff, parts["norm2b"], run_ff)
 
 
 def norm_for(ops, norm, reader, x, out, rows=None):

@@ -64,31 +64,53 @@ class GatedMLP(Part):
 @register_part("feed_forward", "mlp")
 class PlainMLP(Part):
     """``x += Wdown act(Wup h)`` without a gate: ``activation`` is ``gelu_erf`` (0.5 z (1 + erf(z / sqrt 2))),
-    ``gelu_tanh`` or ``relu2`` (the square of relu), computed in fp32 on the product's rounded result. ``names``: the
-    two tensors' names after ``prefix`` (keys up, down)."""
+    ``gelu_tanh`` or ``relu2`` (the square of relu), computed in fp32 on the product's rounded result, or ``polynorm``:
+    ``a N(z) + b N(z^2) + c N(z^3) + e`` with the powers taken element by element, ``N`` dividing a token's vector by its
+    root mean square (``eps`` inside the root) and ``(a, b, c, e)`` the tensor ``act``; its sums are fp32 over the product's
+    32-bit result. ``names``: the tensors' names after ``prefix`` (keys up, down, act). ``forward(..., accumulate=False)``
+    writes ``x = ...`` instead of adding."""
     graph_safe = True
+    can_overwrite = True
 
-    def __init__(self, hidden_size, intermediate_size, activation="gelu_erf", prefix="", names=None):
+    def __init__(self, hidden_size, intermediate_size, activation="gelu_erf", prefix="", names=None, eps=None):
         super().__init__(prefix)
-        if activation not in ("gelu_erf", "gelu_tanh", "relu2"):
+        if activation not in ("gelu_erf", "gelu_tanh", "relu2", "polynorm"):
             fail(ENOTSUP, f"mlp: activation '{activation}' is not implemented")
+        if activation == "polynorm" and eps is None:
+            fail(ENOTSUP, "mlp: the activation of normed powers needs the norm's eps")
         self.E, self.F, self.activation = hidden_size, intermediate_size, activation
-        self.names = {"up": "up_proj.weight", "down": "down_proj.weight"}
+        self.eps = None if eps is None else float(eps)
+        self.names = {"up": "up_proj.weight", "down": "down_proj.weight", "act": "act"}
         self.names.update(names or {})
-        self.w_up = self.w_down = None
+        self.w_up = self.w_down = self.coef = None
 
     def param_specs(self):
-        return [ParamSpec(self.prefix + self.names["up"], (self.F, self.E)),
-                ParamSpec(self.prefix + self.names["down"], (self.E, self.F))]
+        specs = [ParamSpec(self.prefix + self.names["up"], (self.F, self.E)),
+                 ParamSpec(self.prefix + self.names["down"], (self.E, self.F))]
+        if self.activation == "polynorm":
+            specs.append(ParamSpec(self.prefix + self.names["act"], (4,), "vector", ("normal", 0.5)))
+        return specs
 
     def bind(self, params, ops):
         self.w_up = params[self.prefix + self.names["up"]]
         self.w_down = params[self.prefix + self.names["down"]]
+        if self.activation == "polynorm":
+            self.coef = params[self.prefix + self.names["act"]].contiguous()
 
-    def forward(self, ops, step, h, x):
+    def forward(self, ops, step, h, x, accumulate=True):
         T = h.shape[0]
         act = ops.scratch("ffn_act", (T, self.F), ops.act_dtype)
-        with ops.section("up"):
-            ops.gemm(h, self.w_up, act, activation=self.activation)
+        if self.activation == "polynorm":
+            z = ops.scratch("ffn_up", (T, self.F), torch.float32)
+            with ops.section("up"):
+                ops.gemm(h, self.w_up, z)
+            with ops.section("ffn_act"):
+                ops.polynorm(z, self.coef, self.eps, act)
+        else:
+            with ops.section("up"):
+                ops.gemm(h, self.w_up, act, activation=self.activation)
         with ops.section("down"):
-            ops.gemm(act, self.w_down, x, accumulate=True, defer=True)
+            if accumulate:
+                ops.gemm(act, self.w_down, x, accumulate=True, defer=True)
+            else:
+                ops.gemm(act, self.w_down, x)

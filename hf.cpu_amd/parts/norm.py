@@ -13,22 +13,29 @@ class RMSNorm(Part):
     can_be_lazy = True          # forward(..., lazy=True) may leave the division to the products that read the output
 
 
-    def __init__(self, size, eps, prefix=""):
+    def __init__(self, size, eps, prefix="", weight="weight"):
+        """The scale is the tensor ``prefix + weight``."""
         super().__init__(prefix)
         self.size = size
         self.eps = float(eps)
+        self.name = prefix + weight
         self.weight = None
 
     def param_specs(self):
-        return [ParamSpec(self.prefix + "weight", (self.size,), "vector", ("one_plus_normal", 0.1))]
+        return [ParamSpec(self.name, (self.size,), "vector", ("one_plus_normal", 0.1))]
 
     def bind(self, params, ops):
-        self.weight = params[self.prefix + "weight"]
+        self.weight = params[self.name]
 
     def forward(self, ops, x, out, rows=None, lazy=False):
         """``out[r] = norm(x[rows[r]])`` (``rows`` None: every row in order). ``lazy``: the caller promises that
         ``out`` is read through ``ops.gemm`` alone (a part that says ``lazy_input_ok``); see ``Ops.rmsnorm``."""
         ops.rmsnorm(x, self.weight, self.eps, out, rows, lazy=lazy)
+
+    def add_into(self, ops, y, x, gate=None, gate_bias=None, scale=1.0, accumulate=True):
+        """``x (+)= scale * norm(y * sigmoid(gate + gate_bias))`` in fp32: the norm of a branch's result ``y`` (fp32) on its
+        way into the stream (``gate`` None: ``y`` as it is)."""
+        ops.rmsnorm_add(y, self.weight, self.eps, x, gate=gate, gate_bias=gate_bias, scale=scale, accumulate=accumulate)
 
 
 @register_part("norm", "layernorm")

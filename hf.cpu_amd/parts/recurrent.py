@@ -1,11 +1,14 @@
-"""Mixers that keep per-request state of fixed size instead of a growing cache: a state-space layer and linear
-attention with a fixed decay. Both walk a request's tokens in order from the state the step before left, with one
-kernel for the recurrence (``Ops.linear_scan``): ``S <- a_t S + k_t (b_t v_t)^T``, ``y_t = S^T q_t + d v_t``."""
+"""Mixers that keep per-request state of fixed size instead of a growing cache: a state-space layer, linear
+attention with a fixed decay, a matrix memory with exponential gates, and the gated delta rule. All walk a request's
+tokens in order from the state the step before left. The first three share one kernel for the recurrence
+(``Ops.linear_scan``): ``S <- a_t S + k_t (b_t v_t)^T``, ``y_t = S^T q_t + d v_t``; the delta rule, whose write depends on
+what the state already holds along the key, has its own (``Ops.delta_scan``). ``side_by_side`` runs two mixers on one
+input and joins their normed results."""
 import torch
 
 from .. import memory
 from ..kernels.ops import Ops
-from ..registry import register_part
+from ..registry import make_part, register_part
 from ..status import EINVAL, fail
 from .base import FixedState, ParamSpec, Part
 
@@ -144,3 +147,219 @@ class LightningAttention(Part):
             ops.group_rmsnorm(o, self.norm_w, self.eps, 1, normed, gate=gate, gate_kind="sigmoid_after")
         with ops.section("lin_wo"):
             ops.gemm(normed, self.w_o, x, accumulate=True, defer=True)
+
+
+@register_part("mixer", "mlstm")
+class MatrixLSTM(Part):
+    """A matrix memory per head with exponential input gates and sigmoid forget gates, kept stable by a running maximum of
+    the gates' logarithms: ``q = Wq h / sqrt(head_dim)``, ``k = Wk h`` (``n_heads`` x ``head_dim``), ``v = Wv h`` (``n_heads`` x
+    ``v_head_dim``); per head ``li = cap tanh((Wi h + bi) / cap)``, ``lf = logsigmoid(cap tanh((Wf h + bf) / cap))``;
+    ``m_t = max(lf + m_(t-1), li)`` with ``m_0 = 0``; ``S_t = exp(lf + m_(t-1) - m_t) S_(t-1) + exp(li - m_t) k v^T``, ``n_t`` alike
+    with ``k`` alone; ``o_t = S_t^T q / (max(|n_t . q|, exp(-m_t)) + 1e-6)``. Each head's ``o`` is divided by its root mean square
+    (``eps``), the heads together are multiplied by ``norm`` and by ``sigmoid(Wg h)``, and projected. The state (S, n and m of
+    every head), the gates and the recurrence are fp32. ``names``: the tensors' names after ``prefix`` (keys q, k, v, g, o,
+    norm, i, i_bias, f, f_bias). ``forward(..., accumulate=False)`` writes ``x = ...`` instead of adding."""
+    graph_safe = True
+    can_overwrite = True
+
+    def __init__(self, hidden_size, n_heads, head_dim, v_head_dim, gate_cap, eps, prefix="", names=None):
+        super().__init__(prefix)
+        if not gate_cap > 0.0:
+            fail(EINVAL, f"mlstm: the gates' cap {gate_cap} must be positive")
+        self.E, self.H, self.D, self.Dv = hidden_size, n_heads, head_dim, v_head_dim
+        self.cap, self.eps = float(gate_cap), float(eps)
+        self.names = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "g": "g_proj.weight", "o": "out_proj.weight",
+                      "norm": "norm.weight", "i": "i_proj.weight", "i_bias": "i_proj.bias", "f": "f_proj.weight", "f_bias": "f_proj.bias"}
+        self.names.update(names or {})
+        self.w_in = self.w_gates = self.w_o = self.norm_w = self.i_bias = self.f_bias = None
+
+    def param_specs(self):
+        p, nm = self.prefix, self.names
+        QD, VD = self.H * self.D, self.H * self.Dv
+        return [ParamSpec(p + nm["q"], (QD, self.E)), ParamSpec(p + nm["k"], (QD, self.E)), ParamSpec(p + nm["v"], (VD, self.E)),
+                ParamSpec(p + nm["g"], (VD, self.E)), ParamSpec(p + nm["o"], (self.E, VD)),
+                ParamSpec(p + nm["norm"], (VD,), "vector", ("one_plus_normal", 0.1)),
+                ParamSpec(p + nm["i"], (self.H, self.E)), ParamSpec(p + nm["i_bias"], (self.H,), "vector", ("normal", 0.5)),
+                ParamSpec(p + nm["f"], (self.H, self.E)), ParamSpec(p + nm["f_bias"], (self.H,), "vector", ("normal", 0.5))]
+
+    def cache_need(self):
+        return FixedState(Ops.scan_state_floats(self.H, self.D, self.Dv, normalizer=True))
+
+    def bind(self, params, ops):
+        p, nm = self.prefix, self.names
+        mats = [params[p + nm[n]] for n in "qkvg"]
+        dt = torch.float32 if any(m.dtype == torch.float32 for m in mats) else mats[0].dtype
+        self.w_in = memory.cat([m.to(dt) for m in mats], 0, f"{p}q, k, v and the output gate in one matrix")
+        gates = [params[p + nm["i"]], params[p + nm["f"]]]
+        self.w_gates = memory.cat([m.to(dt) for m in gates], 0, f"{p}both gates in one matrix")
+        self.w_o, self.norm_w = params[p + nm["o"]], params[p + nm["norm"]]
+        self.i_bias, self.f_bias = params[p + nm["i_bias"]].contiguous(), params[p + nm["f_bias"]].contiguous()
+
+    def forward(self, ops, step, h, cache, x, write_cache=True, accumulate=True):
+        if not write_cache:
+            fail(EINVAL, f"mlstm '{self.prefix}': a state cannot be read without being advanced")
+        T, QD, VD, H = h.shape[0], self.H * self.D, self.H * self.Dv, self.H
+        proj = ops.scratch("mlstm_in", (T, 2 * QD + 2 * VD), ops.act_dtype)
+        gates = ops.scratch("mlstm_gates", (T, 2 * H), torch.float32)
+        with ops.section("mlstm_in"):
+            ops.gemm(h, self.w_in, proj)
+            ops.gemm(h, self.w_gates, gates)
+        o = ops.scratch("mlstm_o", (T, VD), torch.float32)
+        denom = ops.scratch("mlstm_denom", (T, H), torch.float32)
+        with ops.section("mlstm_scan"):
+            ops.linear_scan(proj[:, :QD], proj[:, QD:2 * QD], proj[:, 2 * QD:2 * QD + VD], H, self.D, H, self.Dv, cache.state, step, o,
+                            exp_gates=(gates[:, :H], gates[:, H:], self.i_bias, self.f_bias, self.cap), q_scale=self.D ** -0.5,
+                            denom=denom)
+        normed = ops.scratch("mlstm_normed", (T, VD), ops.act_dtype)
+        with ops.section("mlstm_norm"):
+            ops.group_rmsnorm(o, self.norm_w, self.eps, H, normed, gate=proj[:, 2 * QD + VD:], gate_kind="sigmoid_after",
+                              row_scale=denom)
+        with ops.section("mlstm_wo"):
+            if accumulate:
+                ops.gemm(normed, self.w_o, x, accumulate=True, defer=True)
+            else:
+                ops.gemm(normed, self.w_o, x)
+
+
+@register_part("mixer", "gated_delta")
+class GatedDelta(Part):
+    """The gated delta rule: ``q = Wq h``, ``k = Wk h`` (``n_qk_heads`` x ``head_dim``), ``v = Wv h`` (``n_heads`` x ``v_head_dim``);
+    each passes a causal convolution over ``conv_taps`` tokens per channel (no bias, zeros before a sequence's start) and
+    silu; ``q`` and ``k`` are made unit vectors head by head (``x / sqrt(sum x^2 + 1e-6)``) and ``q`` is divided by
+    ``sqrt(head_dim)``. Per head h (queries and keys of head ``h // (n_heads / n_qk_heads)``): a write strength
+    ``beta = sigmoid(Wb h)``, a decay per key channel ``g = exp(-exp(A_log_h) softplus(Wa2 (Wa1 h) + dt_bias))``, and
+    ``S <- g * S`` (row by row); ``u = beta (v - S^T k)``; ``S <- S + k u^T``; ``o = S^T q``, so the read-out sees the token's
+    own write. Each head's ``o`` is RMS-normed over ``v_head_dim`` with a weight of that size which all heads share, multiplied
+    by ``sigmoid(Wg2 (Wg1 h))`` and projected. The state (S of every head and the convolution's last ``conv_taps - 1`` inputs),
+    decays, strengths, unit vectors and the recurrence are fp32. ``names``: the tensors' names after ``prefix`` (keys q, k, v,
+    q_conv, k_conv, v_conv, b, a1, a2, dt_bias, a_log, g1, g2, norm, o). ``forward(..., accumulate=False)`` writes ``x = ...``."""
+    graph_safe = True
+    can_overwrite = True
+    UNIT_EPS = 1e-6
+
+    def __init__(self, hidden_size, n_heads, n_qk_heads, head_dim, v_head_dim, conv_taps, eps, decay_rank=None, gate_rank=None,
+                 prefix="", names=None):
+        """``decay_rank`` and ``gate_rank``: the inner sizes of the two low-rank projections (None: taken from the tensors)."""
+        super().__init__(prefix)
+        if n_heads % n_qk_heads:
+            fail(EINVAL, f"gated_delta: {n_heads} heads are not a multiple of {n_qk_heads} heads of queries and keys")
+        if not 1 <= conv_taps <= 8:
+            fail(EINVAL, f"gated_delta: a convolution over {conv_taps} tokens (1 to 8)")
+        self.E, self.H, self.G, self.N, self.P, self.K = hidden_size, n_heads, n_qk_heads, head_dim, v_head_dim, conv_taps
+        self.eps = float(eps)
+        self.ra, self.rg = decay_rank, gate_rank
+        self.KD, self.VD = n_qk_heads * head_dim, n_heads * v_head_dim
+        self.C = 2 * self.KD + self.VD
+        self.n_scan = Ops.scan_state_floats(n_heads, head_dim, v_head_dim)
+        self.names = {n: n for n in ("q", "k", "v", "b", "a1", "a2", "dt_bias", "g1", "g2", "norm", "o")}
+        self.names.update(q_conv="q.conv", k_conv="k.conv", v_conv="v.conv", a_log="A_log")
+        self.names.update(names or {})
+        self.w_qkv = self.w_small = self.w_a2 = self.w_g2 = self.w_o = self.taps = self.dt_bias = self.a_log = self.norm_w = None
+
+    def param_specs(self):
+        p, nm = self.prefix, self.names
+        ra, rg = self.ra or 0, self.rg or 0              # 0: any size (the loader takes the tensor's)
+        return [ParamSpec(p + nm["q"], (self.KD, self.E)), ParamSpec(p + nm["k"], (self.KD, self.E)), ParamSpec(p + nm["v"], (self.VD, self.E)),
+                ParamSpec(p + nm["q_conv"], (self.KD, self.K), "vector", ("normal", 0.3)),
+                ParamSpec(p + nm["k_conv"], (self.KD, self.K), "vector", ("normal", 0.3)),
+                ParamSpec(p + nm["v_conv"], (self.VD, self.K), "vector", ("normal", 0.3)),
+                ParamSpec(p + nm["b"], (self.H, self.E)),
+                ParamSpec(p + nm["a1"], (ra, self.E)), ParamSpec(p + nm["a2"], (self.H * self.N, ra), "matrix", ("normal", 0.1)),
+                ParamSpec(p + nm["dt_bias"], (self.H * self.N,), "vector", ("normal", 0.5)),
+                ParamSpec(p + nm["a_log"], (self.H,), "vector", ("normal", 0.5)),
+                ParamSpec(p + nm["g1"], (rg, self.E)), ParamSpec(p + nm["g2"], (self.VD, rg), "matrix", ("normal", 0.1)),
+                ParamSpec(p + nm["norm"], (self.P,), "vector", ("one_plus_normal", 0.1)),
+                ParamSpec(p + nm["o"], (self.E, self.VD))]
+
+    def cache_need(self):
+        return FixedState(self.n_scan + (self.K - 1) * self.C)
+
+    def bind(self, params, ops):
+        p, nm = self.prefix, self.names
+        mats = [params[p + nm[n]] for n in "qkv"]
+        dt = torch.float32 if any(m.dtype == torch.float32 for m in mats) else mats[0].dtype
+        self.w_qkv = memory.cat([m.to(dt) for m in mats], 0, f"{p}q, k and v in one matrix")
+        small = [params[p + nm[n]] for n in ("b", "a1", "g1")]
+        self.w_small = memory.cat([m.to(dt) for m in small], 0, f"{p}write strength and the low-rank inputs in one matrix")
+        self.ra, self.rg = small[1].shape[0], small[2].shape[0]
+        self.w_a2, self.w_g2, self.w_o = params[p + nm["a2"]], params[p + nm["g2"]], params[p + nm["o"]]
+        if self.w_a2.shape[1] != self.ra or self.w_g2.shape[1] != self.rg:
+            fail(EINVAL, f"gated_delta '{p}': the low-rank projections' inner sizes do not match")
+        self.taps = memory.cat([params[p + nm[n + "_conv"]] for n in "qkv"], 0, f"{p}taps of q, k and v in one matrix").contiguous()
+        self.dt_bias, self.a_log = params[p + nm["dt_bias"]].contiguous(), params[p + nm["a_log"]].contiguous()
+        self.norm_w = memory.cat([params[p + nm["norm"]]] * self.H, 0, f"{p}the heads' norm weight, once a head")
+
+    def forward(self, ops, step, h, cache, x, write_cache=True, accumulate=True):
+        if not write_cache:
+            fail(EINVAL, f"gated_delta '{self.prefix}': a state cannot be read without being advanced")
+        T, KD, VD, H = h.shape[0], self.KD, self.VD, self.H
+        proj = ops.scratch("delta_in", (T, self.C), ops.act_dtype)
+        small = ops.scratch("delta_small", (T, H + self.ra + self.rg), torch.float32)
+        with ops.section("delta_in"):
+            ops.gemm(h, self.w_qkv, proj)
+            ops.gemm(h, self.w_small, small)
+        a = ops.scratch("delta_decay", (T, H * self.N), torch.float32)
+        gate = ops.scratch("delta_gate", (T, VD), ops.act_dtype)
+        with ops.section("delta_low_rank"):
+            ops.gemm(small[:, H:H + self.ra], self.w_a2, a)
+            ops.gemm(small[:, H + self.ra:], self.w_g2, gate)
+        conv = ops.scratch("delta_conv", (T, self.C), torch.float32)
+        with ops.section("delta_conv"):
+            ops.causal_conv(proj, self.taps, None, cache.state[:, self.n_scan:], step, conv, activation="silu")
+        y = ops.scratch("delta_y", (T, VD), torch.float32)
+        with ops.section("delta_scan"):
+            ops.delta_scan(conv[:, :KD], conv[:, KD:2 * KD], conv[:, 2 * KD:], self.G, self.N, H, self.P, a, self.dt_bias, self.a_log,
+                           small[:, :H], cache.state, step, y, q_scale=self.N ** -0.5, unit_eps=self.UNIT_EPS)
+        normed = ops.scratch("delta_normed", (T, VD), ops.act_dtype)
+        with ops.section("delta_norm"):
+            ops.group_rmsnorm(y, self.norm_w, self.eps, H, normed, gate=gate, gate_kind="sigmoid_after")
+        with ops.section("delta_wo"):
+            if accumulate:
+                ops.gemm(normed, self.w_o, x, accumulate=True, defer=True)
+            else:
+                ops.gemm(normed, self.w_o, x)
+
+
+@register_part("mixer", "side_by_side")
+class SideBySide(Part):
+    """Two mixers that read the same input; the result is ``scale * (norm_l(left(h)) + norm_r(right(h)))``, each side RMS-normed
+    over the model's width with a weight of its own (``names``: keys left_norm, right_norm, after ``prefix``) before the sum
+    (``scale`` 0.5: half the sum). ``left`` and ``right`` are PartSpecs of mixers; their caches are this mixer's, by the names
+    ``left`` and ``right``. The sides' results, the norms and the sum are fp32."""
+    graph_safe = True
+    can_overwrite = True
+
+    def __init__(self, hidden_size, left, right, eps, scale=0.5, prefix="", names=None):
+        super().__init__(prefix)
+        self.E, self.eps, self.scale = hidden_size, float(eps), float(scale)
+        self.left, self.right = make_part("mixer", left), make_part("mixer", right)
+        self.names = {"left_norm": "left.out", "right_norm": "right.out"}
+        self.names.update(names or {})
+        self.w_left = self.w_right = None
+        self.short_request_rows = 0
+
+    def sub_parts(self):
+        return [self.left, self.right]
+
+    def param_specs(self):
+        return [ParamSpec(self.prefix + self.names[n], (self.E,), "vector", ("one_plus_normal", 0.1)) for n in ("left_norm", "right_norm")]
+
+    def cache_need(self):
+        return {"left": self.left.cache_need(), "right": self.right.cache_need()}
+
+    def bind(self, params, ops):
+        self.w_left, self.w_right = params[self.prefix + self.names["left_norm"]], params[self.prefix + self.names["right_norm"]]
+        self.short_request_rows = max(getattr(self.left, "short_request_rows", 0), getattr(self.right, "short_request_rows", 0))
+
+    def forward(self, ops, step, h, cache, x, write_cache=True, accumulate=True):
+        T = h.shape[0]
+        for side, w, name in ((self.left, self.w_left, "left"), (self.right, self.w_right, "right")):
+            y = ops.scratch("side_" + name, (T, self.E), torch.float32)
+            if getattr(side, "can_overwrite", False):
+                side.forward(ops, step, h, cache[name], y, write_cache, accumulate=False)
+            else:
+                ops.settle()
+                y.zero_()
+                side.forward(ops, step, h, cache[name], y, write_cache)
+            with ops.section("side_norm"):
+                ops.rmsnorm_add(y, w, self.eps, x, scale=self.scale, accumulate=accumulate or name == "right")

@@ -33,7 +33,7 @@ def check_tensors(entries, specs, origin):
         e = entries.get(s.name)
         if e is None:
             continue
-        if tuple(e.shape) != tuple(s.shape):
+        if len(e.shape) != len(s.shape) or any(want and got != want for got, want in zip(e.shape, s.shape)):   # 0: any size
             shapes.append(f"{s.name} has shape {'x'.join(map(str, e.shape)) or 'scalar'}, "
                           f"expected {'x'.join(map(str, s.shape))}")     # src/model.c:80-82
         allowed = INT_STORED if s.kind == "table" else FLOAT_STORED

@@ -97,6 +97,14 @@ def random_tensor(spec, seed, index, dtype):
     return t if rule == "table" else t.to(dtype)
 
 
+def _sizes_known(specs):
+    """Random weights need every size: a spec that leaves one to the checkpoint (a 0 in its shape) is refused."""
+    from ..status import EINVAL, fail
+    open_ = [s.name for s in specs if not s.optional and any(d == 0 for d in s.shape)]
+    if open_:
+        fail(EINVAL, f"random weights: the configuration leaves sizes of {', '.join(open_[:4])} to a checkpoint's tensors; give them")
+
+
 def write_random_model(model_dir, config, seed, dtype="float32"):
     """Writes ``config.json`` and ``model.safetensors`` for ``config`` (a typed
     configuration of a registered architecture). Optional tensors (a tied head) are
@@ -109,6 +117,7 @@ def write_random_model(model_dir, config, seed, dtype="float32"):
     with open(os.path.join(model_dir, "config.json"), "w") as f:
         json.dump(obj, f, indent=1)
     specs = [s for s in Model.from_config(config).param_specs() if not s.optional]
+    _sizes_known(specs)
     tensors = {}
     for i, s in enumerate(specs):
         dt = torch.int32 if s.kind == "table" else stored
@@ -127,6 +136,7 @@ def random_device_tensors(specs, seed, compute_dtype, device, ops=None):
     from ..status import EINVAL, EngineError
     from .loader import held_dtype
     lib = library()
+    _sizes_known(specs)
     stream = torch.cuda.current_stream(device).cuda_stream
     code = {torch.float32: 0, torch.bfloat16: 1, torch.int32: 2}
     out = {}
