@@ -1,6 +1,6 @@
-"""``bench.py --design goridra | tobozen``: prefill and decode of a design at sizes that resemble a real model's layers
+"""``bench.py --design goridra | tobozen | mobupel``: prefill and decode of a design at sizes that resemble a real model's layers
 (random weights), beside the closest other design at equal width, heads and layer count (Goridra beside Qwen2 dense,
-Tobozen beside Goridra), with every part of a step priced against its roofline: flops / time against the matrix cores
+Tobozen beside Goridra, Mobupel beside Tobozen), with every part of a step priced against its roofline: flops / time against the matrix cores
 for a prefill's parts, bytes / time against HBM for a decode step's. One JSON line a size."""
 import json
 import math
@@ -62,6 +62,42 @@ def tobozen_work(z, T, batch, ctx):
     return pre, dec
 
 
+def mobupel_shape(z):
+    """Layers in pairs: two mixers side by side (softmax attention with mixed heads; the gated delta rule) with a dense
+    feed-forward, then a matrix memory with exponential gates and no feed-forward."""
+    H, G, D, W = z["heads"], z["kv_heads"], z["dim"], z["width"]
+    pair = [
+        dict(type="parallel", mixer=dict(
+            left=dict(heads=H, kv_heads=G, dim=D, vdim=D, scale=1.0 / math.sqrt(D), conv=4),
+            right=dict(heads=H, kv_heads=H, dim=D, vdim=D, conv=4, decay_rank=W // 32, gate_rank=W // 32)), mlp=dict(kind="dense", ff=z["ff"])),
+        dict(type="mlstm", mixer=dict(heads=H, dim=D, vdim=D, gate_cap=15.0), mlp=None)]
+    return dict(architecture="Mobupel", vocab=z["vocab"], width=W, embedding=dict(scale=math.sqrt(W)), logit_scale=1.0, norm=dict(eps=1e-6),
+                layers=pair * (3 * z["triples"] // 2))
+
+
+def mobupel_work(z, T, batch, ctx):
+    """({part: flops of a prefill of T tokens}, {part: bytes of a decode step}), all layers together, bf16. Attention with
+    mixed heads is priced as its scores once and its weights applied to the values of every group (what the identity that
+    the kernels use costs); the recurrences by the products of their state updates and outputs (4 N P a head and token; the
+    delta rule's correction is another 2 N P) in a prefill and by their fp32 states, read and written once a request, in a
+    decode step."""
+    W, H, G, D, V, F = z["width"], z["heads"], z["kv_heads"], z["dim"], z["vocab"], z["ff"]
+    n2 = 3 * z["triples"] // 2
+    QD, KD, r = H * D, G * D, W // 32
+    params = {"qkv": n2 * W * (QD + 2 * KD + QD), "wo": n2 * QD * W, "delta_in": n2 * W * (3 * QD + H + 2 * r),
+              "delta_low_rank": n2 * r * 2 * QD, "delta_wo": n2 * QD * W, "mlstm_in": n2 * W * (4 * QD + 2 * H), "mlstm_wo": n2 * QD * W,
+              "gate": 3 * n2 * W * W, "up": n2 * F * W, "down": n2 * F * W, "head": V * W}
+    pre = {k: 2.0 * T * v for k, v in params.items() if k != "head"}
+    pre["attn"] = n2 * (2.0 + 2.0 * G) * D * H * T * (T + 1) / 2
+    pre["delta_scan"] = n2 * T * H * 6.0 * D * D
+    pre["mlstm_scan"] = n2 * T * H * 4.0 * D * (D + 1)
+    dec = {k: 2.0 * v for k, v in params.items()}
+    dec["attn"] = batch * ctx * 2 * KD * n2 * 2.0
+    dec["delta_scan"] = batch * n2 * H * D * D * 4 * 2.0
+    dec["mlstm_scan"] = batch * n2 * H * D * (D + 1) * 4 * 2.0
+    return pre, dec
+
+
 def goridra_shape(z):
     """Layers in pairs: one with keys and values of its own and a dense feed-forward, one that reads them and has
     a mixture of experts."""
@@ -96,6 +132,8 @@ def part_work(design, z, T, batch, ctx):
     all layers together, bf16."""
     if design == "tobozen":
         return tobozen_work(z, T, batch, ctx)
+    if design == "mobupel":
+        return mobupel_work(z, T, batch, ctx)
     W, H, G, D, L, V = z["width"], z["heads"], z["kv_heads"], z["dim"], z["layers"], z["vocab"]
     QD, KD = H * D, G * D
     if design == "qwen2":
@@ -132,9 +170,9 @@ def run(args):
     for size in (args.sizes.split(",") if args.sizes else list(SIZES)):
         z = SIZES[size]
         line = {"size": size, "dims": z, "context": context, "dtype": "bf16", "data": "synthetic"}
-        shapes = {"goridra": goridra_shape, "qwen2": qwen2_shape, "tobozen": tobozen_shape}
-        beside = {"goridra": "qwen2", "tobozen": "goridra"}[args.design]
-        if args.design == "tobozen":                 # the same number of layers in both designs
+        shapes = {"goridra": goridra_shape, "qwen2": qwen2_shape, "tobozen": tobozen_shape, "mobupel": mobupel_shape}
+        beside = {"goridra": "qwen2", "tobozen": "goridra", "mobupel": "tobozen"}[args.design]
+        if args.design in ("tobozen", "mobupel"):    # the same number of layers in both designs
             z = dict(z, layers=3 * z["triples"])
         for design, shape in ((args.design, shapes[args.design](z)), (beside, shapes[beside](z))):
             cfg = hf_cpu_amd.config_from_dict(shape)

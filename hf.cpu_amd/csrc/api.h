@@ -98,7 +98,7 @@ int hfa_attention_prompt_rows(void);
 // becomes dot * scale + slopes[h] * (j - p); with slopes the plain kernel runs. `sink` 1: the softmax has one more term
 // of score 0 that has no value, p_j = exp(s_j) / (1 + sum_i exp(s_i)) (every kernel takes it). `cross_values` 1: every
 // head's weights are applied to the values of every key/value group: out is [token][G rounds][H heads][v_head_dim], round r
-// of head h being its weights on the values of group (h's group + r) mod G (see hfa_talk_mix; the plain kernel runs).
+// of head h being its weights on the values of group (h's group + r) mod G (see hfa_talk_mix; on the matrix cores one pass a round).
 int hfa_paged_attention(const void* q, int dtype, int ldq, const void* k_cache, const void* v_cache,
                         int kv_width, int v_width, const int* block_table, int max_blocks, const int* token_slot,
                         const int* positions, const int* q_start, int n_seqs, int max_q_len, int max_seq_len,

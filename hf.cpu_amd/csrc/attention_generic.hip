@@ -193,7 +193,7 @@ extern "C" int hfa_decode_attention(const float* raw, int ld_raw, const float* c
                 "decode_attention: a row stride is smaller than its row");
     AttnArgs a = {nullptr, 8, k_cache, v_cache, kv_width, block_table, max_blocks, token_slot, positions, q_start,
                   n_seqs, 1, max_seq_len, out, ldo, n_seqs, n_heads, n_kv_heads, head_dim, page_tokens,
-                  window, scale, workspace, workspace_bytes, stream, raw, ld_raw, cos_sin, slot_map, mask_chunk, 0};
+                  window, scale, workspace, workspace_bytes, stream, raw, ld_raw, cos_sin, slot_map, mask_chunk, 0, 0};
     HFA_REQUIRE(((uintptr_t)raw & 15) == 0 && (cos_sin == nullptr || ((uintptr_t)cos_sin & 15) == 0) && attn_mfma_supports(a),
                 "decode_attention: this shape is not taken (see hfa_decode_attention_supports)");
     return attn_mfma_launch(a);
@@ -217,11 +217,23 @@ extern "C" int hfa_paged_attention(const void* q, int dtype, int ldq, const void
     HFA_REQUIRE(dtype == HFA_F32 || dtype == HFA_BF16, "paged_attention: unknown dtype %d", dtype);
     AttnArgs a = {q, ldq, k_cache, v_cache, kv_width, block_table, max_blocks, token_slot, positions, q_start,
                   n_seqs, max_q_len, max_seq_len, out, ldo, n_tokens, n_heads, n_kv_heads, head_dim, page_tokens,
-                  window, scale, workspace, workspace_bytes, stream, nullptr, 0, nullptr, nullptr, mask_chunk, sink ? 1 : 0};
+                  window, scale, workspace, workspace_bytes, stream, nullptr, 0, nullptr, nullptr, mask_chunk, sink ? 1 : 0, 0};
     // the matrix-core kernels take no slopes: scores with a position term go the plain way
     // and they know one head size and one row width for keys and values
-    if (!force_plain && !slopes && !cross_values && dtype == HFA_BF16 && v_head_dim == head_dim && v_width == kv_width && attn_mfma_supports(a))
-        return attn_mfma_launch(a);
+    if (!force_plain && !slopes && dtype == HFA_BF16 && v_head_dim == head_dim && v_width == kv_width && attn_mfma_supports(a)) {
+        if (!cross_values) return attn_mfma_launch(a);
+        // The weights on every group's values, on the matrix cores: one pass a round, the scores taken again each time (a
+        // round's output lies n_heads * head_dim further on in the token's row, whose stride ldo spans all rounds). The
+        // passes share the workspace; they run one after the other on the stream.
+        for (int r = 0; r < n_kv_heads; r++) {
+            AttnArgs b = a;
+            b.v_rot = r;
+            b.out = (char*)out + (size_t)r * n_heads * head_dim * 2;
+            const int rc = attn_mfma_launch(b);
+            if (rc) return rc;
+        }
+        return 0;
+    }
     return attn_generic_launch(q, dtype, ldq, k_cache, v_cache, kv_width, v_width, block_table, max_blocks, token_slot,
                                positions, out, ldo, n_tokens, n_heads, n_kv_heads, head_dim, v_head_dim, page_tokens, window,
                                mask_chunk, scale, slopes, sink ? 1 : 0, cross_values ? 1 : 0, stream);

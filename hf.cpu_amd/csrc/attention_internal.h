@@ -20,6 +20,7 @@ struct AttnArgs {
     const int* slot_map;           // the cache row of each token's key and value
     int mask_chunk;                // > 0: a query sees only the keys of its own run of mask_chunk positions, counted from 0
     int sink;                      // 1: the softmax's denominator holds one more term of score 0 that has no value
+    int v_rot;                     // the weights of a head of group c are applied to the values of group (c + v_rot) mod G (0: its own)
 };
 
 // The first key that the query at `pos` sees: a window of the last `window` positions (0: none) and/or the start

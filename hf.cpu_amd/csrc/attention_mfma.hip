@@ -78,11 +78,14 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
     const int* __restrict__ positions, const int* __restrict__ q_start, int n_seqs, uint16_t* __restrict__ out,
     int ldo, float* __restrict__ partial, int H, int psh, int window, int mask_chunk, float scale_log2e, int tpt, int cpt,
     int chunk_keys, int n_chunks, int one_tile_each, const float* __restrict__ raw, int ld_raw,
-    const float* __restrict__ cs, const int* __restrict__ slot_map, int G, int sink) {
+    const float* __restrict__ cs, const int* __restrict__ slot_map, int G, int sink, int v_rot) {
     constexpr int D = NDB * 32, KS = D / 16;
     const int P = 1 << psh;                                // tokens per page, a power of two
     const int lane = threadIdx.x, col = lane & 31, half = lane >> 5;
     const int g = blockIdx.y, chunk = blockIdx.z;
+    // The group whose values the weights are applied to: the heads' own, or (v_rot > 0, never with FUSED) the group
+    // v_rot further on, for designs that mix the heads' weights after the softmax (see hfa_talk_mix).
+    const int gv = g + v_rot < G ? g + v_rot : g + v_rot - G;
 
     // ---- the tile's request and tokens: tiles are numbered request by request ----
     int tile = blockIdx.x, t0 = -1, t_end = 0;
@@ -265,7 +268,7 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
                 ka = ka < (hi & ~3) ? ka : (hi & ~3);       // runs past the end are masked; read a valid one
                 const int page = page_of(ka);
                 // element offsets fit 32 bits (checked on the host), so one base serves every load
-                const unsigned off = __umul24((unsigned)(page << psh), (unsigned)kvw) + (unsigned)(((g * D + col) << psh) + (ka & (P - 1)));
+                const unsigned off = __umul24((unsigned)(page << psh), (unsigned)kvw) + (unsigned)(((gv * D + col) << psh) + (ka & (P - 1)));
 #pragma unroll
                 for (int db = 0; db < NDB; db++)
                     vf[db][kk].h[run] = *reinterpret_cast<const uint2*>(vc + (off + (unsigned)((db * 32) << psh)));
@@ -485,7 +488,7 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_slot,
     const int* __restrict__ positions, const int* __restrict__ q_start, int n_seqs, uint16_t* __restrict__ out,
     int ldo, int psh, int window, int mask_chunk, float scale_log2e, int tpt, int cpt, int n_tiles, int pair_from,
-    float* __restrict__ partial, int H, int chunk_keys, int n_chunks, int sink) {
+    float* __restrict__ partial, int H, int chunk_keys, int n_chunks, int sink, int v_rot) {
     constexpr int D = NDB * 32, KS = D / 16, KROW = D + 8;
     const int P = 1 << psh;                                // tokens per page, a power of two
     __shared__ __attribute__((aligned(16))) uint16_t k_s[2][KB * KROW];
@@ -511,6 +514,8 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
             g = j % (int)gridDim.x;
         }
     }
+    // the group whose values the weights are applied to (see attn_mfma_kernel)
+    const int gv = g + v_rot < (int)gridDim.x ? g + v_rot : g + v_rot - (int)gridDim.x;
     int t0 = -1, t_end = 0;
     for (int s = 0; s < n_seqs; s++) {
         const int a = q_start[s], b = q_start[s + 1];
@@ -592,7 +597,7 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
         k_pg[i] = row >> psh;
         k_at[i] = (unsigned)((row & (P - 1)) * kvw + g * D + (c % (D / 8)) * 8);
         v_pg[i] = k8 >> psh;
-        v_at[i] = (unsigned)(((g * D + c / 4) << psh) + (k8 & (P - 1)));
+        v_at[i] = (unsigned)(((gv * D + c / 4) << psh) + (k8 & (P - 1)));
     }
     auto gload = [&](int key0, u32x4 (&rk)[NCH], uint2 (&rv)[NCH][2]) {
         if constexpr (small_pages) {
@@ -622,7 +627,7 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
                 int ka = key0 + 8 * (c % 4);
                 ka = ka < (hi & ~7) ? ka : (hi & ~7);
                 const int page = page_of(ka);
-                const unsigned off = __umul24((unsigned)(page << psh), (unsigned)kvw) + (unsigned)(((g * D + c / 4) << psh) + (ka & (P - 1)));
+                const unsigned off = __umul24((unsigned)(page << psh), (unsigned)kvw) + (unsigned)(((gv * D + c / 4) << psh) + (ka & (P - 1)));
                 const uint4 v = *reinterpret_cast<const uint4*>(vc + off);
                 rv[i][0] = make_uint2(v.x, v.y);
                 rv[i][1] = make_uint2(v.z, v.w);
@@ -894,7 +899,7 @@ static int launch_ndb(const AttnArgs& a, int tiles, int tpt, int cpt, int chunk_
     (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width, a.block_table,      \
         a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo, PARTIAL, a.n_heads,         \
         page_shift(a.page_tokens), a.window, a.mask_chunk, sl, tpt, cpt, chunk_keys, n_chunks, a.max_q_len <= tpt, a.raw, a.ld_raw,      \
-        a.cos_sin, a.slot_map, a.n_kv_heads, a.sink
+        a.cos_sin, a.slot_map, a.n_kv_heads, a.sink, a.v_rot
     if (a.raw) {
         if (n_chunks > 1) attn_mfma_kernel<NDB, true, true><<<grid, WAVE, 0, a.stream>>>(ATTN_ARGS((float*)a.workspace));
         else attn_mfma_kernel<NDB, false, true><<<grid, WAVE, 0, a.stream>>>(ATTN_ARGS(nullptr));
@@ -954,13 +959,13 @@ static int launch_prefill(const AttnArgs& a, int tpt, int cpt) {
             (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width, a.block_table,
             a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo,
             page_shift(a.page_tokens), a.window, a.mask_chunk, a.scale * 1.4426950408889634f, tpt, cpt, n_tiles, pair_from,
-            (float*)a.workspace, a.n_heads, chunk_keys, n_chunks, a.sink);
+            (float*)a.workspace, a.n_heads, chunk_keys, n_chunks, a.sink, a.v_rot);
     else
         attn_prefill_kernel<NDB, false><<<grid, 4 * WAVE, 0, a.stream>>>(
             (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width, a.block_table,
             a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo,
             page_shift(a.page_tokens), a.window, a.mask_chunk, a.scale * 1.4426950408889634f, tpt, cpt, n_tiles, pair_from,
-            (float*)a.workspace, a.n_heads, chunk_keys, n_chunks, a.sink);
+            (float*)a.workspace, a.n_heads, chunk_keys, n_chunks, a.sink, a.v_rot);
     HFA_LAUNCH_CHECK("attn_prefill");
     if (n_chunks > 1) {
         attn_merge_kernel<<<dim3(a.n_tokens, a.n_heads), WAVE, 0, a.stream>>>((const float*)a.workspace, (uint16_t*)a.out, a.ldo,

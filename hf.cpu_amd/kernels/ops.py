@@ -658,7 +658,7 @@ class Ops:
         _ints(step.q_start, "q_start", step.n_seqs + 1)
         # the matrix-core kernels address the cache with 32-bit element offsets and 24-bit row numbers
         too_large = cache.k.numel() >= 1 << 32 or cache.k.shape[0] >= 1 << 24
-        plain = self.force_plain_attention or slopes is not None or too_large or bool(cross_values)
+        plain = self.force_plain_attention or slopes is not None or too_large
         if cross_values and out.shape[1] != n_kv_heads * n_heads * v_head_dim:
             fail(EINVAL, "paged_attention: with cross_values the output holds groups * heads * v_head_dim columns")
         if too_large and q.dtype == torch.bfloat16 and not self._said_cache_too_large:

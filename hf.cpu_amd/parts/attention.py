@@ -38,10 +38,10 @@ class Attention(Part):
     ``names``) and the kept values of the same token; the blended values are what is cached. A ``"first"`` layer holds the
     scalar too, unused.
 
-    ``conv_taps`` K > 1: q, k and v pass a causal convolution over the last K tokens per channel straight after the
+    ``conv_taps`` K >= 1: q, k and v pass a causal convolution over the last K tokens per channel straight after the
     projection (tensors ``q_conv``, ``k_conv``, ``v_conv`` in ``names``, [channels, K], the last column the current token's, no
     bias, zeros before a sequence's start); the last K - 1 projected rows of a request are part of its state, so the mixer
-    then needs ``{"kv": PagedKV, "conv": FixedState}``. ``head_norm`` = eps: queries and keys are RMS-normed head by head over
+    then needs ``{"kv": PagedKV, "conv": FixedState}`` (one tap is a factor per channel and needs no state). ``head_norm`` = eps: queries and keys are RMS-normed head by head over
     ``head_dim`` with weights of that size which all heads share (``q_norm``, ``k_norm``). ``talk``: the heads' softmax weights
     are mixed after the softmax, ``weight_h <- sum_g talk[h, g] weight_g`` (tensor ``talk`` [heads, heads]), and head h applies
     its mixed weights to the values of its own group. ``out_gate``: the concatenated heads are multiplied by
@@ -80,14 +80,14 @@ class Attention(Part):
         self.conv_taps = int(conv_taps)
         self.head_norm = None if head_norm is None else float(head_norm)
         self.talk, self.out_gate = bool(talk), bool(out_gate)
-        self.shaped = self.conv_taps > 1 or self.head_norm is not None or self.talk or self.out_gate
+        self.shaped = self.conv_taps >= 1 or self.head_norm is not None or self.talk or self.out_gate
         if self.shaped and (position.kind != "none" or not own_kv or qk_norm is not None or sink or v_mix or qkv_bias or window
                             or mask_chunk):
             fail(EINVAL, "attention: a convolution, per-head norms, mixed heads and an output gate go without rotation, biases, "
                          "windows and the other options")
         if not 0 <= self.conv_taps <= 8:
             fail(EINVAL, f"attention: a convolution over {self.conv_taps} tokens (at most 8)")
-        self.taps = self.talk_w = None
+        self.taps = self.talk_w = self.no_state = None
         self.qk_norm = None if qk_norm is None else float(qk_norm)
         self.sink = bool(sink)
         if v_mix not in (None, "first", "blend") or (v_mix and not own_kv):
@@ -118,7 +118,7 @@ class Attention(Part):
                 specs.append(ParamSpec(p + nm["k_norm"], (self.KD,), "vector", ("one_plus_normal", 0.1)))
         if self.v_mix:
             specs.append(ParamSpec(p + nm["v_mix"], (), "vector", ("normal", 0.3), optional=self.v_mix == "first"))
-        if self.conv_taps > 1:
+        if self.conv_taps >= 1:
             specs += [ParamSpec(p + nm[n + "_conv"], (widths[n], self.conv_taps), "vector", ("normal", 0.3)) for n in "qkv"]
         if self.head_norm is not None:
             specs += [ParamSpec(p + nm[n], (self.D,), "vector", ("one_plus_normal", 0.1)) for n in ("q_norm", "k_norm")]
@@ -164,7 +164,8 @@ class Attention(Part):
             self.k_norm_w = params[p + nm["k_norm"]] if self.own_kv else None
         if self.v_mix == "blend":
             self.v_blend = params[p + nm["v_mix"]].reshape(1)
-        if self.conv_taps > 1:
+        if self.conv_taps >= 1:
+            self.no_state = memory.zeros((1, 1), torch.float32, ops.device, f"{p}a convolution's state that is never read")
             self.taps = memory.cat([params[p + nm[n + "_conv"]] for n in "qkv"], 0, f"{p}taps of q, k and v in one matrix").contiguous()
         if self.head_norm is not None:
             self.q_norm_w, self.k_norm_w = params[p + nm["q_norm"]].contiguous(), params[p + nm["k_norm"]].contiguous()
@@ -183,9 +184,9 @@ class Attention(Part):
             ops.gemm(h, self.w_qkv, proj)
         rows = proj[:, :C]
         with ops.section("qkv_prepare"):
-            if self.conv_taps > 1:
+            if self.conv_taps >= 1:
                 rows = ops.scratch("qkv_conv", (T, C), torch.float32)
-                ops.causal_conv(proj[:, :C], self.taps, None, cache["conv"].state, step, rows)
+                ops.causal_conv(proj[:, :C], self.taps, None, cache["conv"].state if self.conv_taps > 1 else self.no_state, step, rows)
             q = ops.scratch("q_normed", (T, self.QD), ops.act_dtype)
             ops.head_norm_store(rows, self.H, self.G, self.D, self.Dv, self.q_norm_w, self.k_norm_w, self.head_norm or 0.0, q, kv,
                                 step.group(kv.group).slot_map)

@@ -254,7 +254,7 @@ class GatedDelta(Part):
         self.names = {n: n for n in ("q", "k", "v", "b", "a1", "a2", "dt_bias", "g1", "g2", "norm", "o")}
         self.names.update(q_conv="q.conv", k_conv="k.conv", v_conv="v.conv", a_log="A_log")
         self.names.update(names or {})
-        self.w_qkv = self.w_small = self.w_a2 = self.w_g2 = self.w_o = self.taps = self.dt_bias = self.a_log = self.norm_w = None
+        self.w_qkv = self.w_small = self.w_b = self.w_a2 = self.w_g2 = self.w_o = self.taps = self.dt_bias = self.a_log = self.norm_w = None
 
     def param_specs(self):
         p, nm = self.prefix, self.names
@@ -279,9 +279,10 @@ class GatedDelta(Part):
         mats = [params[p + nm[n]] for n in "qkv"]
         dt = torch.float32 if any(m.dtype == torch.float32 for m in mats) else mats[0].dtype
         self.w_qkv = memory.cat([m.to(dt) for m in mats], 0, f"{p}q, k and v in one matrix")
-        small = [params[p + nm[n]] for n in ("b", "a1", "g1")]
-        self.w_small = memory.cat([m.to(dt) for m in small], 0, f"{p}write strength and the low-rank inputs in one matrix")
-        self.ra, self.rg = small[1].shape[0], small[2].shape[0]
+        small = [params[p + nm[n]] for n in ("a1", "g1")]
+        self.w_small = memory.cat([m.to(dt) for m in small], 0, f"{p}the low-rank projections' first halves in one matrix")
+        self.w_b = params[p + nm["b"]]
+        self.ra, self.rg = small[0].shape[0], small[1].shape[0]
         self.w_a2, self.w_g2, self.w_o = params[p + nm["a2"]], params[p + nm["g2"]], params[p + nm["o"]]
         if self.w_a2.shape[1] != self.ra or self.w_g2.shape[1] != self.rg:
             fail(EINVAL, f"gated_delta '{p}': the low-rank projections' inner sizes do not match")
@@ -294,22 +295,24 @@ class GatedDelta(Part):
             fail(EINVAL, f"gated_delta '{self.prefix}': a state cannot be read without being advanced")
         T, KD, VD, H = h.shape[0], self.KD, self.VD, self.H
         proj = ops.scratch("delta_in", (T, self.C), ops.act_dtype)
-        small = ops.scratch("delta_small", (T, H + self.ra + self.rg), torch.float32)
+        small = ops.scratch("delta_small", (T, self.ra + self.rg), ops.act_dtype)
+        beta = ops.scratch("delta_beta", (T, H), torch.float32)
         with ops.section("delta_in"):
             ops.gemm(h, self.w_qkv, proj)
             ops.gemm(h, self.w_small, small)
+            ops.gemm(h, self.w_b, beta)
         a = ops.scratch("delta_decay", (T, H * self.N), torch.float32)
         gate = ops.scratch("delta_gate", (T, VD), ops.act_dtype)
         with ops.section("delta_low_rank"):
-            ops.gemm(small[:, H:H + self.ra], self.w_a2, a)
-            ops.gemm(small[:, H + self.ra:], self.w_g2, gate)
+            ops.gemm(small[:, :self.ra], self.w_a2, a)
+            ops.gemm(small[:, self.ra:], self.w_g2, gate)
         conv = ops.scratch("delta_conv", (T, self.C), torch.float32)
         with ops.section("delta_conv"):
             ops.causal_conv(proj, self.taps, None, cache.state[:, self.n_scan:], step, conv, activation="silu")
         y = ops.scratch("delta_y", (T, VD), torch.float32)
         with ops.section("delta_scan"):
             ops.delta_scan(conv[:, :KD], conv[:, KD:2 * KD], conv[:, 2 * KD:], self.G, self.N, H, self.P, a, self.dt_bias, self.a_log,
-                           small[:, :H], cache.state, step, y, q_scale=self.N ** -0.5, unit_eps=self.UNIT_EPS)
+                           beta, cache.state, step, y, q_scale=self.N ** -0.5, unit_eps=self.UNIT_EPS)
         normed = ops.scratch("delta_normed", (T, VD), ops.act_dtype)
         with ops.section("delta_norm"):
             ops.group_rmsnorm(y, self.norm_w, self.eps, H, normed, gate=gate, gate_kind="sigmoid_after")
