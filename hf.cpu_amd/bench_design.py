@@ -177,8 +177,9 @@ def run(args):
         for design, shape in ((args.design, shapes[args.design](z)), (beside, shapes[beside](z))):
             cfg = hf_cpu_amd.config_from_dict(shape)
             batches = [int(b) for b in args.batches.split(",")]
-            s = S.Session(cfg, dtype="bfloat16", ctx_max=context + 64, batch=PROMPT, page_size=PAGE, max_seqs=max(batches),
-                          kv_tokens=max(batches) * (context + 64), seed=0)
+            room = -(-(args.steps + 16) // 64) * 64          # the decoded tokens: six to warm up, the timed ones, four profiled
+            s = S.Session(cfg, dtype="bfloat16", ctx_max=context + room, batch=PROMPT, page_size=PAGE, max_seqs=max(batches),
+                          kv_tokens=max(batches) * (context + room), seed=0)
             eng, ops = s.engine, s.ops
 
             def prompt(n=PROMPT):
