@@ -222,6 +222,9 @@ extern "C" int hfa_paged_attention(const void* q, int dtype, int ldq, const void
     // and they know one head size and one row width for keys and values
     if (!force_plain && !slopes && dtype == HFA_BF16 && v_head_dim == head_dim && v_width == kv_width && attn_mfma_supports(a)) {
         if (!cross_values) return attn_mfma_launch(a);
+        // single tokens: one pass over the cache for all rounds
+        int chunk_keys = 0, n_chunks = 0;
+        if (attn_cross_supports(a, &chunk_keys, &n_chunks)) return attn_cross_launch(a, chunk_keys, n_chunks);
         // The weights on every group's values, on the matrix cores: one pass a round, the scores taken again each time (a
         // round's output lies n_heads * head_dim further on in the token's row, whose stride ldo spans all rounds). The
         // passes share the workspace; they run one after the other on the stream.

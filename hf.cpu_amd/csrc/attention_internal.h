@@ -39,6 +39,12 @@ int attn_generic_launch(const void* q, int dtype, int ldq, const void* k_cache, 
                         void* out, int ldo, int n_tokens, int n_heads, int n_kv_heads, int head_dim, int v_head_dim,
                         int page_tokens, int window, int mask_chunk, float scale, const float* slopes, int sink, int cross, hipStream_t stream);
 
+// Single tokens of a mixer that mixes its heads' weights after the softmax: every head's weights on the values of every
+// group in one pass over the cache, written in rounds of groups (see attention_cross.hip). `supports` leaves the cut
+// of the keys that `launch` takes.
+bool attn_cross_supports(const AttnArgs& a, int* chunk_keys, int* n_chunks);
+int attn_cross_launch(const AttnArgs& a, int chunk_keys, int n_chunks);
+
 // bf16 on the matrix cores; see attention_mfma.hip for what it needs.
 bool attn_mfma_supports(const AttnArgs& a);
 int attn_mfma_launch(const AttnArgs& a);

@@ -228,22 +228,25 @@ extern "C" int hfa_head_norm_store(const void* qkv, int in_dtype, int ld, int n_
 // values of group c. `cross` holds these: [T][G rounds][H heads][Dv], round r of head g being its weights on the values
 // of group (c(g) + r) mod G (hfa_paged_attention with cross_values). gate (null: none): out is multiplied by
 // sigmoid(gate[t, h Dv + d]). Sums in fp32 in the order of g.
+// A block a (token, head): with few tokens (a decode step) there are still heads x tokens blocks to fill the machine.
 template <typename TA, typename TG, typename TO>
-__global__ __launch_bounds__(256) void talk_mix_kernel(const TA* __restrict__ cross, const float* __restrict__ talk,
+__global__ __launch_bounds__(128) void talk_mix_kernel(const TA* __restrict__ cross, const float* __restrict__ talk,
                                                       const TG* __restrict__ gate, int ldg, TO* __restrict__ out, int ldo, int H,
                                                       int G, int Dv) {
-    extern __shared__ float talk_s[];
-    const int t = blockIdx.x, per = H / G;
-    for (int i = threadIdx.x; i < H * H; i += blockDim.x) talk_s[i] = talk[i];
+    extern __shared__ float talk_s[];                      // row h of the mix, and where each head's round for h's group lies
+    int* at_s = reinterpret_cast<int*>(talk_s + H);
+    const int t = blockIdx.x, h = blockIdx.y, per = H / G, c = h / per;
+    for (int g = threadIdx.x; g < H; g += blockDim.x) {
+        talk_s[g] = talk[h * H + g];
+        at_s[g] = (((c - g / per + G) % G) * H + g) * Dv;
+    }
     __syncthreads();
     const TA* A = cross + (size_t)t * G * H * Dv;
-    for (int i = threadIdx.x; i < H * Dv; i += blockDim.x) {
-        const int h = i / Dv, d = i % Dv, c = h / per;
+    for (int d = threadIdx.x; d < Dv; d += blockDim.x) {
         float acc = 0.f;
-        for (int g = 0; g < H; g++) {
-            const int r = (c - g / per + G) % G;
-            acc = fmaf(talk_s[h * H + g], to_f32(A[((size_t)r * H + g) * Dv + d]), acc);
-        }
+#pragma unroll 4
+        for (int g = 0; g < H; g++) acc = fmaf(talk_s[g], to_f32(A[at_s[g] + d]), acc);
+        const int i = h * Dv + d;
         if (gate) acc *= 1.0f / (1.0f + expf(-to_f32(gate[(size_t)t * ldg + i])));
         out[(size_t)t * ldo + i] = from_f32<TO>(acc);
     }
@@ -255,10 +258,10 @@ extern "C" int hfa_talk_mix(const void* cross, int cross_dtype, const float* tal
                 "talk_mix: bad arguments");
     HFA_REQUIRE(n_heads <= 128, "talk_mix: %d heads (at most 128)", n_heads);
     HFA_REQUIRE(ldo >= n_heads * v_head_dim && (!gate || ldg >= n_heads * v_head_dim), "talk_mix: a row is shorter than its heads");
-    const size_t lds = (size_t)n_heads * n_heads * sizeof(float);
+    const size_t lds = (size_t)n_heads * (sizeof(float) + sizeof(int));
     const int code = (cross_dtype == HFA_BF16 ? 4 : 0) + ((gate && gate_dtype == HFA_BF16) ? 2 : 0) + (out_dtype == HFA_BF16 ? 1 : 0);
 #define TM(TA, TG, TO)                                                                                                          \
-    talk_mix_kernel<TA, TG, TO><<<n_tokens, 256, lds, stream>>>((const TA*)cross, talk, (const TG*)gate, ldg, (TO*)out, ldo, n_heads, \
+    talk_mix_kernel<TA, TG, TO><<<dim3(n_tokens, n_heads), 128, lds, stream>>>((const TA*)cross, talk, (const TG*)gate, ldg, (TO*)out, ldo, n_heads, \
                                                                 n_kv_heads, v_head_dim)
     switch (code) {
         case 0: TM(float, float, float); break;

@@ -194,7 +194,8 @@ def paged_kv(rng, lengths, G, D, Dv, page, dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,G,D,Dv,page", [(6, 3, 10, 6, 8), (4, 4, 8, 12, 4), (8, 2, 64, 64, 16), (4, 1, 32, 32, 16), (6, 2, 128, 128, 32),
-                                           (8, 4, 96, 96, 16), (5, 5, 48, 48, 16), (3, 1, 64, 24, 16)])
+                                           (8, 4, 96, 96, 16), (5, 5, 48, 48, 16), (3, 1, 64, 24, 16), (6, 3, 64, 64, 8), (32, 2, 32, 32, 4), (9, 3, 128, 128, 64),
+                                           (16, 8, 64, 64, 16), (12, 6, 32, 32, 8), (32, 8, 128, 128, 16)])
 def test_attention_weights_mixed_across_heads(ops32, ops16, dtype, H, G, D, Dv, page):
     """Portions of prompts and single tokens at the end of requests of many lengths, one of them long enough that a decoded
     token's keys are cut over several waves; in each request one query's head and one far key are scaled so that this key
@@ -214,6 +215,8 @@ def test_attention_weights_mixed_across_heads(ops32, ops16, dtype, H, G, D, Dv, 
             q_full[n - 1, 1] = ks[s][far, g] * (12.0 / scale / float(ks[s][far, g] @ ks[s][far, g]))
             pg = table[s, far // page]
             kc[pg * page + far % page] = ks[s][far].reshape(-1)
+            sc = scale * (ks[s][:, g].astype(np.float64) @ q_full[n - 1, 1].astype(np.float64))
+            assert np.exp(sc[far] - sc.max()) / np.exp(sc - sc.max()).sum() > 0.5, "the far key was meant to stand out"
         full = pm.talking_attention(rounded(q_full, dtype), rounded(ks[s], dtype), rounded(vs[s], dtype), scale, talk.astype(np.float64))
         qs.append(q_full[n - ql:])
         wants.append(full[n - ql:])
@@ -238,9 +241,14 @@ def test_attention_weights_mixed_across_heads(ops32, ops16, dtype, H, G, D, Dv, 
         assert np.max(np.abs(out.float().cpu().numpy() - want)) <= tol, f"plain={plain_kernel}"
         ops.talk_mix(cross, dev(talk), H, G, Dv, out, gate=dev(gate_rows, dtype)[:, 16:])
         assert np.max(np.abs(out.float().cpu().numpy() - want * pm.sigmoid(gate_rows[:, 16:]))) <= tol, f"plain={plain_kernel}"
-    # the far key carries the weight it was given: without it the last row of a long request changes by far more than rounding
-    last = sum(q_lens[:5]) - 1
-    assert np.max(np.abs(want[last])) > 10 * tol
+    # single tokens alone (a decode step): in bf16, where the sizes allow, one pass over the cache for all groups' values
+    ends = np.cumsum(q_lens) - 1
+    step1 = FakeStep(ints([n - 1 for n in lengths]), ints(list(range(len(lengths)))), ints(table), None)
+    cross = torch.empty((len(lengths), G * H * Dv), dtype=dtype, device="cuda")
+    ops.paged_attention(dev(q[ends], dtype), H, G, D, cache, step1, 0, scale, cross, v_head_dim=Dv, cross_values=True)
+    out = torch.empty((len(lengths), H * Dv), dtype=dtype, device="cuda")
+    ops.talk_mix(cross, dev(talk), H, G, Dv, out)
+    assert np.max(np.abs(out.float().cpu().numpy() - want[ends])) <= tol, "single tokens"
 
 
 def scan_in_portions(q, cuts, slots, n_state, call):
