@@ -72,7 +72,7 @@ def mobupel_shape(z):
             right=dict(heads=H, kv_heads=H, dim=D, vdim=D, conv=4, decay_rank=W // 32, gate_rank=W // 32)), mlp=dict(kind="dense", ff=z["ff"])),
         dict(type="mlstm", mixer=dict(heads=H, dim=D, vdim=D, gate_cap=15.0), mlp=None)]
     return dict(architecture="Mobupel", vocab=z["vocab"], width=W, embedding=dict(scale=math.sqrt(W)), logit_scale=1.0, norm=dict(eps=1e-6),
-                layers=pair * (3 * z["triples"] // 2))
+                layers=(pair * (3 * z["triples"]))[:3 * z["triples"]])
 
 
 def mobupel_work(z, T, batch, ctx):
@@ -82,19 +82,20 @@ def mobupel_work(z, T, batch, ctx):
     delta rule's correction is another 2 N P) in a prefill and by their fp32 states, read and written once a request, in a
     decode step."""
     W, H, G, D, V, F = z["width"], z["heads"], z["kv_heads"], z["dim"], z["vocab"], z["ff"]
-    n2 = 3 * z["triples"] // 2
+    L = 3 * z["triples"]
+    n2, n1 = (L + 1) // 2, L // 2                      # layers with two mixers side by side and a feed-forward; layers with a matrix memory
     QD, KD, r = H * D, G * D, W // 32
     params = {"qkv": n2 * W * (QD + 2 * KD + QD), "wo": n2 * QD * W, "delta_in": n2 * W * (3 * QD + H + 2 * r),
-              "delta_low_rank": n2 * r * 2 * QD, "delta_wo": n2 * QD * W, "mlstm_in": n2 * W * (4 * QD + 2 * H), "mlstm_wo": n2 * QD * W,
-              "gate": 3 * n2 * W * W, "up": n2 * F * W, "down": n2 * F * W, "head": V * W}
+              "delta_low_rank": n2 * r * 2 * QD, "delta_wo": n2 * QD * W, "mlstm_in": n1 * W * (4 * QD + 2 * H), "mlstm_wo": n1 * QD * W,
+              "gate": (2 * n2 + n1) * W * W, "up": n2 * F * W, "down": n2 * F * W, "head": V * W}
     pre = {k: 2.0 * T * v for k, v in params.items() if k != "head"}
     pre["attn"] = n2 * (2.0 + 2.0 * G) * D * H * T * (T + 1) / 2
     pre["delta_scan"] = n2 * T * H * 6.0 * D * D
-    pre["mlstm_scan"] = n2 * T * H * 4.0 * D * (D + 1)
+    pre["mlstm_scan"] = n1 * T * H * 4.0 * D * (D + 1)
     dec = {k: 2.0 * v for k, v in params.items()}
     dec["attn"] = batch * ctx * 2 * KD * n2 * 2.0
     dec["delta_scan"] = batch * n2 * H * D * D * 4 * 2.0
-    dec["mlstm_scan"] = batch * n2 * H * D * (D + 1) * 4 * 2.0
+    dec["mlstm_scan"] = batch * n1 * H * D * (D + 1) * 4 * 2.0
     return pre, dec
 
 
