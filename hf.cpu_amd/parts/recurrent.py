@@ -228,8 +228,8 @@ class GatedDelta(Part):
     silu; ``q`` and ``k`` are made unit vectors head by head (``x / sqrt(sum x^2 + 1e-6)``) and ``q`` is divided by
     ``sqrt(head_dim)``. Per head h (queries and keys of head ``h // (n_heads / n_qk_heads)``): a write strength
     ``beta = sigmoid(Wb h)``, a decay per key channel ``g = exp(-exp(A_log_h) softplus(Wa2 (Wa1 h) + dt_bias))``, and
-    ``S <- g * S`` (row by row); ``u = beta (v - S^T k)``; ``S <- S + k u^T``; ``o = S^T q``, so the read-out sees the token's
-    own write. Each head's ``o`` is RMS-normed over ``v_head_dim`` with a weight of that size which all heads share, multiplied
+    ``S <- g * S`` (row by row); ``u = beta (v - S^T k)``; ``S <- S + k u^T``; ``o = S^T q``: a token is read
+    from the state that already holds it. Each head's ``o`` is RMS-normed over ``v_head_dim`` with a weight of that size which all heads share, multiplied
     by ``sigmoid(Wg2 (Wg1 h))`` and projected. The state (S of every head and the convolution's last ``conv_taps - 1`` inputs),
     decays, strengths, unit vectors and the recurrence are fp32. ``names``: the tensors' names after ``prefix`` (keys q, k, v,
     q_conv, k_conv, v_conv, b, a1, a2, dt_bias, a_log, g1, g2, norm, o). ``forward(..., accumulate=False)`` writes ``x = ...``."""

@@ -68,8 +68,8 @@ def test_matrix_memory_against_its_sum_form():
                 n += a * k[s, h]
             want = S.T @ q[t, h] / (max(abs(n @ q[t, h]), 1.0) + 1e-6 * math.exp(m))
             assert np.allclose(got[t, h], want)
-    # the running maximum starts at 0, not at minus infinity: a first token whose input gate is far below 0 is
-    # written with the weight exp(i), not 1
+    # m_0 = 0: a first token whose input gate is far below 0 is written with the weight exp(i), where a maximum
+    # that began below every gate would give it the weight 1
     o = pm.mlstm_scan(q[:1], k[:1], v[:1], np.full((1, H), -5.0), np.full((1, H), -0.1))
     for h in range(H):
         assert np.allclose(o[0, h], math.exp(-5.0) * (k[0, h] @ q[0, h]) * v[0, h] / (max(math.exp(-5.0) * abs(k[0, h] @ q[0, h]), 1.0) + 1e-6))
