@@ -113,12 +113,13 @@ extern "C" int hfa_rmsnorm_add(const float* y, int ldy, const void* gate, int ga
 // out = a N(z) + b N(z^2) + c N(z^3) + e over a row, N(u) = u / sqrt(mean(u^2) + eps); coef = (a, b, c, e) on the device.
 // The three sums of squares (of z, z^2 and z^3) are taken in one pass, in fp32, in a fixed order.
 template <typename TI, typename TO>
-__global__ __launch_bounds__(256) void polynorm_kernel(const TI* __restrict__ z, int ldz, const float* __restrict__ coef,
+__global__ __launch_bounds__(1024) void polynorm_kernel(const TI* __restrict__ z, int ldz, const float* __restrict__ coef,
                                                       TO* __restrict__ out, int ldo, int width, float eps) {
     __shared__ float red[17];
     const int r = blockIdx.x;
     const TI* src = z + (size_t)r * ldz;
     float s1 = 0.f, s2 = 0.f, s3 = 0.f;
+#pragma unroll 4
     for (int i = threadIdx.x; i < width; i += blockDim.x) {
         const float v = to_f32(src[i]), v2 = v * v, v3 = v2 * v;
         s1 = fmaf(v, v, s1);
@@ -131,6 +132,7 @@ __global__ __launch_bounds__(256) void polynorm_kernel(const TI* __restrict__ z,
     const float i3 = coef[2] / sqrtf(block_sum(s3, red) / n + eps);
     const float e = coef[3];
     TO* dst = out + (size_t)r * ldo;
+#pragma unroll 4
     for (int i = threadIdx.x; i < width; i += blockDim.x) {
         const float v = to_f32(src[i]), v2 = v * v;
         dst[i] = from_f32<TO>(v * i1 + v2 * i2 + v2 * v * i3 + e);
@@ -141,7 +143,8 @@ extern "C" int hfa_polynorm(const void* z, int z_dtype, int ldz, const float* co
                             int width, float eps, hipStream_t stream) {
     HFA_REQUIRE(z && coef && out && n_rows > 0 && width > 0 && ldz >= width && ldo >= width, "polynorm: bad arguments");
     HFA_REQUIRE((z_dtype == HFA_F32 || z_dtype == HFA_BF16) && (out_dtype == HFA_F32 || out_dtype == HFA_BF16), "polynorm: unknown dtype");
-#define PN(TI, TO) polynorm_kernel<TI, TO><<<n_rows, 256, 0, stream>>>((const TI*)z, ldz, coef, (TO*)out, ldo, width, eps)
+    const int threads = width >= 4096 ? 1024 : 256;       // few rows in a decode step: a wide row is shared by more threads
+#define PN(TI, TO) polynorm_kernel<TI, TO><<<n_rows, threads, 0, stream>>>((const TI*)z, ldz, coef, (TO*)out, ldo, width, eps)
     if (z_dtype == HFA_F32) { if (out_dtype == HFA_F32) PN(float, float); else PN(float, bf16); }
     else { if (out_dtype == HFA_F32) PN(bf16, float); else PN(bf16, bf16); }
 #undef PN
@@ -170,7 +173,8 @@ extern "C" int hfa_scale_rows(float* x, int ld, int n_rows, int width, float s, 
 // Rows [q: H D | k: G D | v: G Dv] (fp32 or bf16): every q head and every k head is divided by sqrt(mean(head^2) + eps) and
 // multiplied by a weight of D values that all heads share (q_w, k_w; null: no norm for that part). q goes to q_out
 // ([T, H D], the cache's dtype), k to cache row slot_map[t], v to the same row with the page transposed
-// ([page][column][offset]). One wave a head, four waves a block, one block a token.
+// ([page][column][offset]). One wave a head, four waves a block, a block a token and four heads; the blocks of a token
+// share its values out.
 template <typename TI, typename TO>
 __global__ __launch_bounds__(256) void head_norm_store_kernel(const TI* __restrict__ qkv, int ld, int H, int G, int D, int Dv,
                                                              const float* __restrict__ q_w, const float* __restrict__ k_w, float eps,
@@ -180,7 +184,8 @@ __global__ __launch_bounds__(256) void head_norm_store_kernel(const TI* __restri
     const TI* row = qkv + (size_t)t * ld;
     const int QD = H * D, KD = G * D, VD = G * Dv;
     const int slot = slot_map[t];
-    for (int hs = wv; hs < H + G; hs += nw) {
+    const int hs = blockIdx.y * nw + wv;
+    if (hs < H + G) {
         const bool is_key = hs >= H;
         const TI* src = row + hs * D;
         const float* w = is_key ? k_w : q_w;
@@ -197,7 +202,7 @@ __global__ __launch_bounds__(256) void head_norm_store_kernel(const TI* __restri
             dst[i] = from_f32<TO>(v);
         }
     }
-    for (int c = threadIdx.x; c < VD; c += blockDim.x)
+    for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < VD; c += gridDim.y * blockDim.x)
         v_cache[(size_t)(slot / page_tokens) * page_tokens * VD + (size_t)c * page_tokens + slot % page_tokens] =
             from_f32<TO>(to_f32(row[QD + KD + c]));
 }
@@ -212,7 +217,7 @@ extern "C" int hfa_head_norm_store(const void* qkv, int in_dtype, int ld, int n_
     HFA_REQUIRE((in_dtype == HFA_F32 || in_dtype == HFA_BF16) && (out_dtype == HFA_F32 || out_dtype == HFA_BF16),
                 "head_norm_store: unknown dtype");
 #define HNS(TI, TO)                                                                                                          \
-    head_norm_store_kernel<TI, TO><<<n_tokens, 256, 0, stream>>>((const TI*)qkv, ld, n_heads, n_kv_heads, head_dim, v_head_dim, \
+    head_norm_store_kernel<TI, TO><<<dim3(n_tokens, (n_heads + n_kv_heads + 3) / 4), 256, 0, stream>>>((const TI*)qkv, ld, n_heads, n_kv_heads, head_dim, v_head_dim, \
                                                                  q_w, k_w, eps, (TO*)q_out, ldq, (TO*)k_cache, (TO*)v_cache,   \
                                                                  slot_map, page_tokens)
     if (in_dtype == HFA_F32) { if (out_dtype == HFA_F32) HNS(float, float); else HNS(float, bf16); }
