@@ -162,7 +162,8 @@ int hfa_qkv_prepare(void* qkv, int dtype, int ld, const int* positions, const fl
 // q_scale multiplies the queries.
 // hfa_delta_scan: the gated delta rule on fp32 inputs, S in hfa_linear_scan's layout: g_t[n] = exp(-exp(a_log[h]) softplus(a[t,
 // h N + n] + dt_bias[h N + n])), S <- g_t * S (row by row), u = sigmoid(b[t, h]) (v_t - S^T k_t), S <- S + k_t u^T, y_t = S^T q_t,
-// with k_t, q_t first divided by sqrt(sum of squares + unit_eps) and q_t multiplied by q_scale.
+// with k_t, q_t first divided by sqrt(sum of squares + unit_eps) and q_t multiplied by q_scale. max_q_len: the most tokens of a
+// request (an upper bound will do; it only chooses between a walk for prompt portions and one for single tokens).
 int hfa_causal_conv(const void* in, int dtype, int ld_in, const float* taps, const float* bias, int n_channels, int n_taps,
                     float* state, size_t state_ld, const int* q_start, const int* seq_slot, int n_seqs, int max_q_len, float* out,
                     int ldo, int act, hipStream_t stream);
@@ -176,7 +177,7 @@ size_t hfa_linear_scan_max_floats(int n_heads, int qk_dim, int v_dim);
 int hfa_delta_scan(const float* q, int ldq, const float* k, int ldk, int qk_heads, int qk_dim, const float* v, int ldv, int n_heads,
                    int v_dim, const float* a, int lda, const float* dt_bias, const float* a_log, const float* b, int ldb,
                    float q_scale, float unit_eps, float* state, size_t state_ld, const int* q_start, const int* seq_slot,
-                   int n_seqs, float* y, int ldy, hipStream_t stream);
+                   int n_seqs, int max_q_len, float* y, int ldy, hipStream_t stream);
 
 // Layers that norm a branch's result before it joins the stream, and what comes with them (sandwich.hip).
 // hfa_embed_pos: x[t] = table[tokens[t]] * scale + pos(positions[t]), pos[2i] = sin(p inv_freq[i]), pos[2i + 1] = cos(p inv_freq[i])

@@ -192,14 +192,25 @@ __global__ __launch_bounds__(SCAN_THREADS) void linear_scan_kernel(
             if (tid < WAVE) {                                   // the maximum runs from token to token: one wave, in order
                 const float li = cap * tanhf((g_.step + sb) * inv_cap), zf = cap * tanhf((g_.step2 + sb2) * inv_cap);
                 const float lf = -(fmaxf(-zf, 0.f) + log1pf(expf(-fabsf(zf))));          // logsigmoid
-                float a_mine = 0.f, b_mine = 0.f, m_mine = 0.f;
-                for (int t = 0; t < TOK && c0 + t < n_tok; t++) {
-                    const float f_t = __shfl(lf, t, WAVE), i_t = __shfl(li, t, WAVE);
-                    const float mn = fmaxf(f_t + m_run, i_t);
-                    if (tid == t) { a_mine = expf(f_t + m_run - mn); b_mine = expf(i_t - mn); m_mine = mn; }
-                    m_run = mn;
+                // only the maximum itself is a chain (an add and a maximum a token, the gates read from their lanes); the
+                // exponentials wait until every lane knows its token's maximum and the one before
+                float m_before = 0.f, m_mine = 0.f;
+#pragma unroll
+                for (int t = 0; t < TOK; t++) {
+                    if (c0 + t < n_tok) {                           // (the same for the whole wave)
+                        const float f_t = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(lf), t));
+                        const float i_t = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(li), t));
+                        const float mn = fmaxf(f_t + m_run, i_t);
+                        if (tid == t) { m_before = m_run; m_mine = mn; }
+                        m_run = mn;
+                    }
                 }
-                if (tid < TOK) { a_s[tid] = a_mine; b_s[tid] = b_mine; m_s[tid] = m_mine; }
+                if (tid < TOK) {
+                    const bool live = c0 + tid < n_tok;
+                    a_s[tid] = live ? expf(lf + m_before - m_mine) : 0.f;
+                    b_s[tid] = live ? expf(li - m_mine) : 0.f;
+                    m_s[tid] = m_mine;
+                }
             }
         } else if (tid < TOK) {
             if (gate == 1) {
@@ -359,7 +370,31 @@ extern "C" int hfa_linear_scan(const void* q, int ldq, const void* k, int ldk, i
 // and every operation are fp32. The block, its lanes and the staging through LDS are linear_scan_kernel's; what differs is
 // that a token's correction needs S^T k_t whole before the state moves, so the lanes of a column add their shares of it
 // across lanes inside the walk (a butterfly: every lane gets the same bits), where that kernel has no traffic at all.
-template <int NS, int NPT>
+// The sum over an aligned run of NS neighbouring lanes (4, 8 or 16: inside a row of the data-parallel primitives), left in
+// every lane of the run with the same bits: neighbours, pairs, then the mirror of a half row and of a row, which pair a
+// lane with one of the other quad or half whose lanes all hold that side's sum already. No trip through LDS: these are
+// modifiers of the adds themselves, and they stand in the chain from one token's state to the next.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float x) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, true));
+}
+template <int NS>
+__device__ __forceinline__ float run_sum(float x) {
+    if constexpr (NS == 4 || NS == 8 || NS == 16) {
+        x += dpp_move<0xB1>(x);                            // quad_perm [1, 0, 3, 2]
+        x += dpp_move<0x4E>(x);                            // quad_perm [2, 3, 0, 1]
+        if constexpr (NS >= 8) x += dpp_move<0x141>(x);    // row_half_mirror
+        if constexpr (NS >= 16) x += dpp_move<0x140>(x);   // row_mirror
+    } else {
+#pragma unroll
+        for (int off = 1; off < NS; off <<= 1) x += __shfl_xor(x, off, WAVE);
+    }
+    return x;
+}
+
+// AHEAD: the walk of whole chunks reads operands ahead (steps with prompt portions); without it the kernel needs fewer
+// registers and more blocks share a compute unit, which is what a step of single tokens lives on.
+template <int NS, int NPT, bool AHEAD>
 __global__ __launch_bounds__(SCAN_THREADS) void delta_scan_kernel(
     const float* __restrict__ q, int ldq, const float* __restrict__ k, int ldk, int heads_per_qk, int N, const float* __restrict__ v,
     int ldv, int P, const float* __restrict__ a, int lda, const float* __restrict__ dt_bias, const float* __restrict__ a_log,
@@ -449,43 +484,68 @@ __global__ __launch_bounds__(SCAN_THREADS) void delta_scan_kernel(
         stash(g_);
         __syncthreads();
         fetch(g_, c0 + 2 * TOK);
-        for (int t = 0; t < nt; t++) {
+        // A token's operands leave LDS two tokens before its multiply-adds (as in linear_scan_kernel): what is left between
+        // one token's state and the next is the decay, the sum over the column's lanes, the correction and the write.
+        struct Operands { float4 k[NPT / 4], q[NPT / 4], g[NPT / 4]; float beta, v; };
+        auto read = [&](int t, Operands& o) {
             const float4* kt = reinterpret_cast<const float4*>(k_s + t * NPAD + ns * NPT);
             const float4* qt = reinterpret_cast<const float4*>(q_s + t * NPAD + ns * NPT);
             const float4* gt = reinterpret_cast<const float4*>(g_s + t * NPAD + ns * NPT);
-            float4 kk[NPT / 4], qq[NPT / 4];
+#pragma unroll
+            for (int i = 0; i < NPT / 4; i++) {
+                o.k[i] = kt[i];
+                o.q[i] = qt[i];
+                o.g[i] = gt[i];
+            }
+            o.beta = b_s[t];
+            o.v = v_s[t * PT + pl];
+        };
+        auto token = [&](int t, const Operands& o) {
             float d0 = 0.f, d1 = 0.f;
 #pragma unroll
             for (int i = 0; i < NPT / 4; i++) {
-                const float4 gg = gt[i];
-                kk[i] = kt[i];
-                qq[i] = qt[i];
+                const float4 gg = o.g[i], kk = o.k[i];
                 st[4 * i] *= gg.x;
                 st[4 * i + 1] *= gg.y;
                 st[4 * i + 2] *= gg.z;
                 st[4 * i + 3] *= gg.w;
-                d0 = fmaf(st[4 * i], kk[i].x, d0);
-                d1 = fmaf(st[4 * i + 1], kk[i].y, d1);
-                d0 = fmaf(st[4 * i + 2], kk[i].z, d0);
-                d1 = fmaf(st[4 * i + 3], kk[i].w, d1);
+                d0 = fmaf(st[4 * i], kk.x, d0);
+                d1 = fmaf(st[4 * i + 1], kk.y, d1);
+                d0 = fmaf(st[4 * i + 2], kk.z, d0);
+                d1 = fmaf(st[4 * i + 3], kk.w, d1);
             }
-            float dot = d0 + d1;
-#pragma unroll
-            for (int off = 1; off < NS; off <<= 1) dot += __shfl_xor(dot, off, WAVE);
-            const float u = b_s[t] * (v_s[t * PT + pl] - dot);
+            const float dot = run_sum<NS>(d0 + d1);
+            const float u = o.beta * (o.v - dot);
             float acc0 = 0.f, acc1 = 0.f;
 #pragma unroll
             for (int i = 0; i < NPT / 4; i++) {
-                st[4 * i] = fmaf(kk[i].x, u, st[4 * i]);
-                st[4 * i + 1] = fmaf(kk[i].y, u, st[4 * i + 1]);
-                st[4 * i + 2] = fmaf(kk[i].z, u, st[4 * i + 2]);
-                st[4 * i + 3] = fmaf(kk[i].w, u, st[4 * i + 3]);
-                acc0 = fmaf(st[4 * i], qq[i].x, acc0);
-                acc1 = fmaf(st[4 * i + 1], qq[i].y, acc1);
-                acc0 = fmaf(st[4 * i + 2], qq[i].z, acc0);
-                acc1 = fmaf(st[4 * i + 3], qq[i].w, acc1);
+                const float4 kk = o.k[i], qq = o.q[i];
+                st[4 * i] = fmaf(kk.x, u, st[4 * i]);
+                st[4 * i + 1] = fmaf(kk.y, u, st[4 * i + 1]);
+                st[4 * i + 2] = fmaf(kk.z, u, st[4 * i + 2]);
+                st[4 * i + 3] = fmaf(kk.w, u, st[4 * i + 3]);
+                acc0 = fmaf(st[4 * i], qq.x, acc0);
+                acc1 = fmaf(st[4 * i + 1], qq.y, acc1);
+                acc0 = fmaf(st[4 * i + 2], qq.z, acc0);
+                acc1 = fmaf(st[4 * i + 3], qq.w, acc1);
             }
             part_s[t * SCAN_THREADS + tid] = acc0 + acc1;
+        };
+        if (AHEAD && nt == TOK) {
+            Operands ring[3];
+            read(0, ring[0]);
+            read(1, ring[1]);
+#pragma unroll
+            for (int t = 0; t < TOK; t++) {
+                if (t + 2 < TOK) read(t + 2, ring[(t + 2) % 3]);
+                token(t, ring[t % 3]);
+            }
+        } else {
+            for (int t = 0; t < nt; t++) {
+                Operands o;
+                read(t, o);
+                token(t, o);
+            }
         }
         __syncthreads();
         for (int idx = tid; idx < nt * PT; idx += SCAN_THREADS) {
@@ -514,7 +574,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void delta_scan_kernel(
 extern "C" int hfa_delta_scan(const float* q, int ldq, const float* k, int ldk, int qk_heads, int qk_dim, const float* v, int ldv,
                               int n_heads, int v_dim, const float* a, int lda, const float* dt_bias, const float* a_log,
                               const float* b, int ldb, float q_scale, float unit_eps, float* state, size_t state_ld,
-                              const int* q_start, const int* seq_slot, int n_seqs, float* y, int ldy, hipStream_t stream) {
+                              const int* q_start, const int* seq_slot, int n_seqs, int max_q_len, float* y, int ldy, hipStream_t stream) {
     HFA_REQUIRE(q && k && v && a && dt_bias && a_log && b && state && q_start && seq_slot && y && n_seqs > 0, "delta_scan: a null argument");
     HFA_REQUIRE(n_heads > 0 && qk_heads > 0 && n_heads % qk_heads == 0 && qk_dim > 0 && v_dim > 0,
                 "delta_scan: %d heads over %d heads of keys", n_heads, qk_heads);
@@ -527,10 +587,13 @@ extern "C" int hfa_delta_scan(const float* q, int ldq, const float* k, int ldk, 
     const int pt = SCAN_THREADS / ns, p_tiles = (v_dim + pt - 1) / pt;
     HFA_REQUIRE(n_heads <= 65535 && n_seqs <= 65535 && p_tiles <= 65535, "delta_scan: the step exceeds the grid");
     dim3 grid(n_heads, n_seqs, p_tiles);
-#define DELTA_GO(NS, NPT)                                                                                                       \
-    delta_scan_kernel<NS, NPT><<<grid, SCAN_THREADS, 0, stream>>>(q, ldq, k, ldk, n_heads / qk_heads, qk_dim, v, ldv, v_dim, a, lda, \
-                                                                  dt_bias, a_log, b, ldb, q_scale, unit_eps, state, state_ld,     \
-                                                                  q_start, seq_slot, y, ldy)
+    const bool ahead = max_q_len >= SCAN_TOKENS;            // some request brings a whole chunk
+#define DELTA_ARGS q, ldq, k, ldk, n_heads / qk_heads, qk_dim, v, ldv, v_dim, a, lda, dt_bias, a_log, b, ldb, q_scale, unit_eps, state, state_ld, q_start, seq_slot, y, ldy
+#define DELTA_GO(NS, NPT)                                                                              \
+    do {                                                                                               \
+        if (ahead) delta_scan_kernel<NS, NPT, true><<<grid, SCAN_THREADS, 0, stream>>>(DELTA_ARGS);   \
+        else delta_scan_kernel<NS, NPT, false><<<grid, SCAN_THREADS, 0, stream>>>(DELTA_ARGS);        \
+    } while (0)
     if (ns == 4) DELTA_GO(4, 4);
     else if (ns == 8 && npt == 4) DELTA_GO(8, 4);
     else if (ns == 8) DELTA_GO(8, 8);
@@ -538,6 +601,7 @@ extern "C" int hfa_delta_scan(const float* q, int ldq, const float* k, int ldk, 
     else if (npt == 8) DELTA_GO(16, 8);
     else DELTA_GO(16, 16);
 #undef DELTA_GO
+#undef DELTA_ARGS
     HFA_LAUNCH_CHECK("delta_scan");
     return 0;
 }

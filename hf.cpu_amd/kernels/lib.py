@@ -23,7 +23,7 @@ _SIGNATURES = {
     "hfa_rope_store": [P, I, I, P, P, I, I, I, I, I, P, P, P, I, I, P, I, P, P],
     "hfa_paged_attention": [P, I, I, P, P, I, I, P, I, P, P, P, I, I, I, P, I, I, I, I, I, I, I, I, I, F, P, I, I, P, c_size_t, I, P],
     "hfa_group_rmsnorm": [P, I, I, P, P, I, I, P, I, I, I, F, P, I, I, I, P, P],
-    "hfa_delta_scan": [P, I, P, I, I, I, P, I, I, I, P, I, P, P, P, I, F, F, P, c_size_t, P, P, I, P, I, P],
+    "hfa_delta_scan": [P, I, P, I, I, I, P, I, I, I, P, I, P, P, P, I, F, F, P, c_size_t, P, P, I, I, P, I, P],
     "hfa_embed_pos": [P, I, P, P, P, P, I, I, I, F, P],
     "hfa_rmsnorm_add": [P, I, P, I, I, P, P, P, I, I, I, F, F, I, P],
     "hfa_polynorm": [P, I, I, P, P, I, I, I, I, F, P],

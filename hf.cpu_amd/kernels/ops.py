@@ -904,7 +904,7 @@ class Ops:
             q.data_ptr(), _rows(q, "scan q"), k.data_ptr(), _rows(k, "scan k"), qk_heads, qk_dim, v.data_ptr(), _rows(v, "scan v"),
             n_heads, v_dim, a.data_ptr(), _rows(a, "scan a"), dt_bias.data_ptr(), a_log.data_ptr(), b.data_ptr(), _rows(b, "scan b"),
             float(q_scale), float(unit_eps), state.data_ptr(), state.stride(0), _ints(step.q_start, "q_start", step.n_seqs + 1),
-            _ints(step.seq_slot, "seq_slot", step.n_seqs), step.n_seqs, y.data_ptr(), _rows(y, "scan out"), self._stream()))
+            _ints(step.seq_slot, "seq_slot", step.n_seqs), step.n_seqs, int(step.max_q_len), y.data_ptr(), _rows(y, "scan out"), self._stream()))
 
     # ---- layer norm, plain activations, soft cap -----------------------------------------------------------------
     def layernorm(self, x, weight, bias, eps, out, rows=None):
