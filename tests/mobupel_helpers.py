@@ -47,9 +47,9 @@ SMALL = config(131, 40, eps=1e-5, embedding_scale=3.0, logit_scale=0.25, layers=
     layer(parallel(left(5, 1, 6, 6, 4, scale=1.0), right(6, 1, 4, 9, 1)), 33),
 ])
 # Sizes that the matrix-core kernels take: attention heads of 64, 32 and 128 whose values have the keys' size, in groups of
-# four, one and two heads; states of 64 x 64, 128 x 32, 32 x 64 and 64 x 128.
+# two, one and two heads; states of 64 x 64, 128 x 32, 32 x 64 and 64 x 128.
 CORES = config(520, 256, layers=[
-    layer(parallel(left(8, 2, 64, 64, 4), right(4, 2, 64, 64, 4)), 384),
+    layer(parallel(left(8, 4, 64, 64, 3), right(4, 2, 64, 64, 4)), 320),
     layer(mlstm(4, 64, 64, 15.0), None),
     layer(parallel(left(4, 4, 32, 32, 2), right(2, 2, 128, 32, 3)), 512),
     layer(mlstm(2, 128, 64, 10.0), 256),
