@@ -6,6 +6,7 @@ from .qwen2 import Qwen2Config
 from .goridra import GoridraConfig
 from .tobozen import TobozenConfig
 from .mobupel import MobupelConfig
+from .gitasun import GitasunConfig
 
 
 def architecture_name(obj, origin="config.json"):
@@ -49,4 +50,4 @@ def read_config(model_dir, options=None):
     return config_from_dict(apply_model_options(read_json_file(path), options, path), path)
 
 
-__all__ = ["GoridraConfig", "KeyReader", "MobupelConfig", "Qwen2Config", "TobozenConfig", "architecture_name", "apply_model_options", "config_from_dict", "read_config", "read_json_file"]
+__all__ = ["GitasunConfig", "GoridraConfig", "KeyReader", "MobupelConfig", "Qwen2Config", "TobozenConfig", "architecture_name", "apply_model_options", "config_from_dict", "read_config", "read_json_file"]

@@ -99,11 +99,15 @@ int hfa_attention_prompt_rows(void);
 // of score 0 that has no value, p_j = exp(s_j) / (1 + sum_i exp(s_i)) (every kernel takes it). `cross_values` 1: every
 // head's weights are applied to the values of every key/value group: out is [token][G rounds][H heads][v_head_dim], round r
 // of head h being its weights on the values of group (h's group + r) mod G (see hfa_talk_mix; on the matrix cores one pass a round).
+// `softcap` > 0: score <- softcap tanh(score / softcap) before the weights are formed. `weights` 0: softmax; 1: no softmax, a
+// visible key weighs sigmoid(score + head_bias[h]) (head_bias: one fp32 per query head, or null), not normalised over the keys.
+// Both go the plain way.
 int hfa_paged_attention(const void* q, int dtype, int ldq, const void* k_cache, const void* v_cache,
                         int kv_width, int v_width, const int* block_table, int max_blocks, const int* token_slot,
                         const int* positions, const int* q_start, int n_seqs, int max_q_len, int max_seq_len,
                         void* out, int ldo, int n_tokens, int n_heads, int n_kv_heads, int head_dim, int v_head_dim,
                         int page_tokens, int window, int mask_chunk, float scale, const float* slopes, int sink, int cross_values,
+                        float softcap, int weights, const float* head_bias,
                         void* workspace, size_t workspace_bytes, int force_plain, hipStream_t stream);
 
 // Decoded tokens (one a request) whose queries, new keys and new values are still the 32-bit rows [q | k | v] that
@@ -131,7 +135,7 @@ int hfa_layernorm(float* x, const float* w, const float* b, void* out, int out_d
 
 // RMS norm in groups: a row of `width` values is cut into `groups` equal runs, each divided by sqrt(mean(run^2) + eps),
 // the whole times w; x and out fp32 or bf16, sums in fp32. rows: out[r] = norm(x[rows[r]]). gate_kind 1: the row is
-// multiplied by silu(gate[r]) before the norm; 2: the result is multiplied by sigmoid(gate[r]) (no rows then). row_scale
+// multiplied by silu(gate[r]) before the norm; 2: the result is multiplied by sigmoid(gate[r]), 3: by silu(gate[r]) (no rows then). row_scale
 // (null: none; fp32 [n_rows, groups], rows in order): run g of row r is multiplied by row_scale[r, g] before everything else.
 int hfa_group_rmsnorm(const void* x, int x_dtype, int ldx, const float* w, void* out, int out_dtype, int ldo, const int* rows,
                       int n_rows, int width, int groups, float eps, const void* gate, int gate_dtype, int ldg, int gate_kind,
@@ -201,6 +205,31 @@ int hfa_head_norm_store(const void* qkv, int in_dtype, int ld, int n_heads, int 
 int hfa_talk_mix(const void* cross, int cross_dtype, const float* talk, const void* gate, int gate_dtype, int ldg, void* out,
                  int out_dtype, int ldo, int n_tokens, int n_heads, int n_kv_heads, int v_head_dim, hipStream_t stream);
 
+// hfa_scale_add: out[r, c] (+)= scale * col[c] * y[r, c] in fp32 (col null: 1). hfa_gate_mul: out = x * act(gate) element by
+// element, formed in fp32; act is HFA_ACT_SIGMOID or HFA_ACT_SILU.
+int hfa_scale_add(const float* y, int ldy, const float* col, float scale, float* out, int ldo, int n_rows, int width,
+                  int accumulate, hipStream_t stream);
+int hfa_gate_mul(const void* x, int x_dtype, int ldx, const void* gate, int gate_dtype, int ldg, void* out, int out_dtype,
+                 int ldo, int n_rows, int width, int act, hipStream_t stream);
+
+// Attention through latents (latent.hip). hfa_latent_pack lays a step's rows out for hfa_rope_store and hfa_paged_attention with one
+// key/value head whose key is [rotated part: R | latent: C] and whose value is the latent: from `down` ([T, >= C + R] fp32: the
+// latent before its norm, then the rotated key part) and `q` ([T, H (D + R)], head by head [D unrotated | R to be rotated]) it
+// writes packed[t] = [H heads of (R | C: left alone) | R | C | C]: the queries' parts to be rotated, the key's part to be rotated,
+// and the latent c = down[:C] / sqrt(mean(down[:C]^2) + eps) * w twice (as the key's rest and as the value). Sums in fp32.
+int hfa_latent_pack(const float* down, int ld_down, const void* q, int q_dtype, int ldq, const float* w, float eps, void* packed,
+                    int out_dtype, int ld_packed, int n_tokens, int n_heads, int dim, int rot, int latent, hipStream_t stream);
+
+// hfa_channel_scan (recurrent.hip): per head, S [qk_dim][v_dim] in hfa_linear_scan's layout: S <- diag(a_t) S + k_t v_t^T, y_t = S^T
+// (q_scale q_t), with a decay per key channel formed in fp32 from gate[t, h qk_dim + n] + gate_bias[h qk_dim + n] = z:
+// form 0: a = lower[h qk_dim + n] + (1 - lower) sigmoid(z), and k_t = 1 - a_t (k is not read);
+// form 1: a = sigmoid(z)^inv_tau = exp(inv_tau logsigmoid(z)), k_t read from k.
+// q_act HFA_ACT_SILU: the queries pass silu first (0: as they are).
+int hfa_channel_scan(const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, int dtype, const void* gate,
+                     int gate_dtype, int ld_gate, const float* gate_bias, int form, const float* lower, float inv_tau, int q_act,
+                     int n_heads, int qk_dim, int v_dim, float q_scale, float* state, size_t state_ld, const int* q_start,
+                     const int* seq_slot, int n_seqs, float* y, int ldy, hipStream_t stream);
+
 // out[r, c] = act(in[r, c]) for rows of `width` values with strides ldi and ldo, computed in fp32:
 // the exact gelu 0.5 z (1 + erf(z / sqrt 2)), its tanh form, relu(z)^2, silu or the logistic function.
 #ifndef HFA_ACT_GELU_ERF
@@ -219,7 +248,8 @@ int hfa_activation(const void* in, int ldi, void* out, int ldo, int dtype, int n
 int hfa_softcap(float* x, int ld, int n_rows, int width, float cap, hipStream_t stream);
 
 // Mixture of experts (moe.hip). hfa_moe_route: fp32 router logits [n_tokens, n_experts] -> ids and weights
-// [n_tokens, top]; scoring 0 = softmax over all experts, 1 = logistic per expert; experts form n_groups equal runs of
+// [n_tokens, top]; scoring 0 = softmax over all experts, 1 = logistic per expert, 2 = exp(logit - largest logit) (with renorm:
+// the softmax over the chosen logits alone); experts form n_groups equal runs of
 // neighbours of which the `keep` best (by their best expert) may be chosen from; weights = score (/ sum of the chosen
 // + 1e-20 if renorm) * out_scale. hfa_moe_plan puts the n_pairs = n_tokens * top pairs in expert order (row_pair) and
 // lists tiles of at most tile_rows rows of one expert (tiles: 3 ints a tile, room for n_pairs / tile_rows + n_experts;

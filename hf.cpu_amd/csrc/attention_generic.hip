@@ -8,6 +8,7 @@
 #include "attention_internal.h"
 
 #define ATT_MAX_D 256
+#define ATT_MAX_D_WIDE 640       // heads that hold a latent and a rotated part side by side
 
 __device__ __forceinline__ float dot_row(const float* __restrict__ q_s, const bf16* __restrict__ kp, int D) {
     float dot = 0.f;
@@ -46,13 +47,16 @@ __device__ __forceinline__ float dot_row(const float* __restrict__ q_s, const fl
 // ATT_MAX_CROSS columns), and out is [token][G rounds][H heads][Dv]: round r of head h holds its weights on the values of
 // group (h's group + r) mod G. A design that mixes the heads' weights after the softmax sums these (hfa_talk_mix).
 #define ATT_MAX_CROSS 1024
-template <typename T, bool CROSS>
+// softcap > 0: score <- softcap tanh(score / softcap). weights 1: no softmax; a visible key weighs sigmoid(score + head_bias[h])
+// (head_bias null: 0), and the weights are not normalised over the keys.
+template <typename T, bool CROSS, int MAXD>
 __global__ __launch_bounds__(WAVE) void attn_generic_kernel(
     const T* __restrict__ q, int ldq, const T* __restrict__ kc, const T* __restrict__ vc, int kvw, int vw,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_slot,
     const int* __restrict__ positions, T* __restrict__ out, int ldo, int H, int G, int D, int Dv, int page_tokens,
-    int window, int mask_chunk, float scale, const float* __restrict__ slopes, int sink) {
-    __shared__ float q_s[ATT_MAX_D];
+    int window, int mask_chunk, float scale, const float* __restrict__ slopes, int sink, float softcap, int weights,
+    const float* __restrict__ head_bias) {
+    __shared__ float q_s[MAXD];
     __shared__ float p_s[WAVE];
     __shared__ int row_s[WAVE];
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
@@ -64,7 +68,9 @@ __global__ __launch_bounds__(WAVE) void attn_generic_kernel(
     const int lo = first_visible(pos, window, mask_chunk);
     const float slope = slopes ? slopes[h] : 0.f;           // a position encoding that enters the scores
     float m = -INFINITY, l = 0.f;
-    constexpr int NACC = (CROSS ? ATT_MAX_CROSS : ATT_MAX_D) / WAVE;
+    constexpr int NACC = (CROSS ? ATT_MAX_CROSS : MAXD) / WAVE;
+    const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
+    const float hb = (weights == 1 && head_bias) ? head_bias[h] : 0.f;
     const int v_first = CROSS ? 0 : kvh * Dv, v_cols = CROSS ? G * Dv : Dv;      // the columns of a value row that this head reads
     float acc[NACC];
 #pragma unroll
@@ -79,13 +85,19 @@ __global__ __launch_bounds__(WAVE) void attn_generic_kernel(
             row = bt[j / page_tokens] * page_tokens + j % page_tokens;
             s = dot_row(q_s, kc + (size_t)row * kvw + kvh * D, D) * scale;
             if (slopes) s += slope * (float)(j - pos);
+            if (softcap > 0.f) s = softcap * tanhf(s * inv_cap);
         }
-        // every tile holds at least one visible key, so the maximum is finite
-        const float mn = fmaxf(m, wave_max(s));
-        const float corr = expf(m - mn);
-        const float p = valid ? expf(s - mn) : 0.f;
-        l = l * corr + wave_sum(p);
-        m = mn;
+        float corr = 1.f, p;
+        if (weights == 1) {
+            p = valid ? 1.0f / (1.0f + expf(-(s + hb))) : 0.f;
+        } else {
+            // every tile holds at least one visible key, so the maximum is finite
+            const float mn = fmaxf(m, wave_max(s));
+            corr = expf(m - mn);
+            p = valid ? expf(s - mn) : 0.f;
+            l = l * corr + wave_sum(p);
+            m = mn;
+        }
         p_s[lane] = p;
         row_s[lane] = row;
         __syncthreads();
@@ -107,7 +119,7 @@ __global__ __launch_bounds__(WAVE) void attn_generic_kernel(
         }
         __syncthreads();
     }
-    const float inv = 1.0f / (sink ? l + expf(-m) : l);      // the term of score 0 that has no value
+    const float inv = weights == 1 ? 1.f : 1.0f / (sink ? l + expf(-m) : l);      // the term of score 0 that has no value
 #pragma unroll
     for (int i = 0; i < NACC; i++) {
         const int d = lane + WAVE * i;
@@ -124,19 +136,23 @@ __global__ __launch_bounds__(WAVE) void attn_generic_kernel(
 int attn_generic_launch(const void* q, int dtype, int ldq, const void* k_cache, const void* v_cache, int kv_width,
                         int v_width, const int* block_table, int max_blocks, const int* token_slot, const int* positions,
                         void* out, int ldo, int n_tokens, int n_heads, int n_kv_heads, int head_dim, int v_head_dim,
-                        int page_tokens, int window, int mask_chunk, float scale, const float* slopes, int sink, int cross, hipStream_t stream) {
+                        int page_tokens, int window, int mask_chunk, float scale, const float* slopes, int sink, int cross, float softcap,
+                        int weights, const float* head_bias, hipStream_t stream) {
     HFA_REQUIRE(!cross || n_kv_heads * v_head_dim <= ATT_MAX_CROSS, "paged_attention: a value row of %d columns exceeds what one wave "
                 "applies its weights to (%d)", n_kv_heads * v_head_dim, ATT_MAX_CROSS);
-    HFA_REQUIRE(head_dim <= ATT_MAX_D && v_head_dim <= ATT_MAX_D, "paged_attention: head_dim %d (values: %d) exceeds the kernel's limit %d",
-                head_dim, v_head_dim, ATT_MAX_D);
+    const bool wide = head_dim > ATT_MAX_D || v_head_dim > ATT_MAX_D;
+    HFA_REQUIRE(head_dim <= ATT_MAX_D_WIDE && v_head_dim <= ATT_MAX_D_WIDE && !(wide && cross),
+                "paged_attention: head_dim %d (values: %d) exceeds the kernel's limit %d", head_dim, v_head_dim, ATT_MAX_D_WIDE);
+    HFA_REQUIRE(weights == 0 || (weights == 1 && !sink), "paged_attention: weights are a softmax (0) or sigmoids without a sink term (1)");
     HFA_REQUIRE(n_heads <= 65535, "paged_attention: %d heads exceed the grid", n_heads);
     dim3 grid(n_tokens, n_heads);
-#define ATT_GO(T, CROSS)                                                                                                          \
-    attn_generic_kernel<T, CROSS><<<grid, WAVE, 0, stream>>>(                                                                     \
+#define ATT_GO(T, CROSS, MAXD)                                                                                                    \
+    attn_generic_kernel<T, CROSS, MAXD><<<grid, WAVE, 0, stream>>>(                                                               \
         (const T*)q, ldq, (const T*)k_cache, (const T*)v_cache, kv_width, v_width, block_table, max_blocks, token_slot, positions, \
-        (T*)out, ldo, n_heads, n_kv_heads, head_dim, v_head_dim, page_tokens, window, mask_chunk, scale, slopes, sink)
-    if (dtype == HFA_F32) { if (cross) ATT_GO(float, true); else ATT_GO(float, false); }
-    else { if (cross) ATT_GO(bf16, true); else ATT_GO(bf16, false); }
+        (T*)out, ldo, n_heads, n_kv_heads, head_dim, v_head_dim, page_tokens, window, mask_chunk, scale, slopes, sink, softcap,   \
+        weights, head_bias)
+    if (dtype == HFA_F32) { if (cross) ATT_GO(float, true, ATT_MAX_D); else if (wide) ATT_GO(float, false, ATT_MAX_D_WIDE); else ATT_GO(float, false, ATT_MAX_D); }
+    else { if (cross) ATT_GO(bf16, true, ATT_MAX_D); else if (wide) ATT_GO(bf16, false, ATT_MAX_D_WIDE); else ATT_GO(bf16, false, ATT_MAX_D); }
 #undef ATT_GO
     HFA_LAUNCH_CHECK("paged_attention");
     return 0;
@@ -204,7 +220,8 @@ extern "C" int hfa_paged_attention(const void* q, int dtype, int ldq, const void
                                    const int* positions, const int* q_start, int n_seqs, int max_q_len,
                                    int max_seq_len, void* out, int ldo, int n_tokens, int n_heads, int n_kv_heads,
                                    int head_dim, int v_head_dim, int page_tokens, int window, int mask_chunk, float scale,
-                                   const float* slopes, int sink, int cross_values, void* workspace, size_t workspace_bytes,
+                                   const float* slopes, int sink, int cross_values, float softcap, int weights,
+                                   const float* head_bias, void* workspace, size_t workspace_bytes,
                                    int force_plain, hipStream_t stream) {
     HFA_REQUIRE(n_tokens > 0 && n_heads > 0 && n_kv_heads > 0 && head_dim > 0 && v_head_dim > 0 && page_tokens > 0 && max_blocks > 0,
                 "paged_attention: bad sizes");
@@ -220,7 +237,9 @@ extern "C" int hfa_paged_attention(const void* q, int dtype, int ldq, const void
                   window, scale, workspace, workspace_bytes, stream, nullptr, 0, nullptr, nullptr, mask_chunk, sink ? 1 : 0, 0};
     // the matrix-core kernels take no slopes: scores with a position term go the plain way
     // and they know one head size and one row width for keys and values
-    if (!force_plain && !slopes && dtype == HFA_BF16 && v_head_dim == head_dim && v_width == kv_width && attn_mfma_supports(a)) {
+    HFA_REQUIRE(softcap >= 0.f && (weights == 0 || weights == 1), "paged_attention: a negative soft cap or an unknown kind of weights");
+    // nor a soft cap on the scores, nor weights that are no softmax
+    if (!force_plain && !slopes && softcap == 0.f && weights == 0 && dtype == HFA_BF16 && v_head_dim == head_dim && v_width == kv_width && attn_mfma_supports(a)) {
         if (!cross_values) return attn_mfma_launch(a);
         // single tokens: one pass over the cache for all rounds
         int chunk_keys = 0, n_chunks = 0;
@@ -239,5 +258,5 @@ extern "C" int hfa_paged_attention(const void* q, int dtype, int ldq, const void
     }
     return attn_generic_launch(q, dtype, ldq, k_cache, v_cache, kv_width, v_width, block_table, max_blocks, token_slot,
                                positions, out, ldo, n_tokens, n_heads, n_kv_heads, head_dim, v_head_dim, page_tokens, window,
-                               mask_chunk, scale, slopes, sink ? 1 : 0, cross_values ? 1 : 0, stream);
+                               mask_chunk, scale, slopes, sink ? 1 : 0, cross_values ? 1 : 0, softcap, weights, head_bias, stream);
 }

@@ -37,7 +37,8 @@ __host__ __device__ __forceinline__ int first_visible(int pos, int window, int m
 int attn_generic_launch(const void* q, int dtype, int ldq, const void* k_cache, const void* v_cache, int kv_width,
                         int v_width, const int* block_table, int max_blocks, const int* token_slot, const int* positions,
                         void* out, int ldo, int n_tokens, int n_heads, int n_kv_heads, int head_dim, int v_head_dim,
-                        int page_tokens, int window, int mask_chunk, float scale, const float* slopes, int sink, int cross, hipStream_t stream);
+                        int page_tokens, int window, int mask_chunk, float scale, const float* slopes, int sink, int cross, float softcap,
+                        int weights, const float* head_bias, hipStream_t stream);
 
 // Single tokens of a mixer that mixes its heads' weights after the softmax: every head's weights on the values of every
 // group in one pass over the cache, written in rounds of groups (see attention_cross.hip). `supports` leaves the cut

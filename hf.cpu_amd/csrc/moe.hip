@@ -28,7 +28,8 @@ __device__ __forceinline__ void wave_best(float& v, int& i) {
     }
 }
 
-// One wave a token. score = softmax over all experts (or the logistic function of each logit, `scoring` 1); experts
+// One wave a token. score = softmax over all experts (or the logistic function of each logit, `scoring` 1; or, `scoring` 2,
+// exp(logit - the largest logit), which with `renorm` makes the weights the softmax over the chosen logits alone); experts
 // form n_groups runs of neighbours, a run scores as its best expert, and only experts of the `keep` best runs can
 // be chosen; the `top` best of those are chosen, and weigh score / (sum of the chosen scores + 1e-20) if `renorm`,
 // else their score; times `out_scale`.
@@ -52,6 +53,11 @@ __global__ __launch_bounds__(WAVE) void moe_route_kernel(const float* __restrict
         }
         sum = wave_sum(sum);
         for (int e = lane; e < E; e += WAVE) s[e] = s[e] / sum;
+    } else if (scoring == 2) {
+        float m = -INFINITY;
+        for (int e = lane; e < E; e += WAVE) m = fmaxf(m, z[e]);
+        m = wave_max(m);
+        for (int e = lane; e < E; e += WAVE) s[e] = expf(z[e] - m);
     } else {
         for (int e = lane; e < E; e += WAVE) s[e] = 1.0f / (1.0f + expf(-z[e]));
     }
@@ -105,7 +111,7 @@ extern "C" int hfa_moe_route(const float* logits, int ld, int n_tokens, int n_ex
     HFA_REQUIRE(top > 0 && top <= WAVE && top <= n_experts, "moe_route: %d choices of %d experts (at most %d)", top, n_experts, WAVE);
     HFA_REQUIRE(n_groups > 0 && n_experts % n_groups == 0 && keep > 0 && keep <= n_groups,
                 "moe_route: %d experts do not form %d equal groups of which %d are kept", n_experts, n_groups, keep);
-    HFA_REQUIRE(scoring == 0 || scoring == 1, "moe_route: unknown scoring %d", scoring);
+    HFA_REQUIRE(scoring >= 0 && scoring <= 2, "moe_route: unknown scoring %d", scoring);
     moe_route_kernel<<<n_tokens, WAVE, 0, stream>>>(logits, ld, n_experts, top, n_groups, keep, scoring, renorm, out_scale, ids,
                                                     weights);
     HFA_LAUNCH_CHECK("moe_route");

@@ -135,7 +135,7 @@ extern "C" int hfa_softcap(float* x, int ld, int n_rows, int width, float cap, h
 // A row of `width` values is cut into `groups` equal runs; each run is divided by sqrt(mean(run^2) + eps) and the
 // whole is multiplied by w (one block a (row, run); sums in fp32 in a fixed order). gate_kind 1: the row is first
 // multiplied by silu(gate) (the gate comes before the norm); gate_kind 2: the normed and weighted row is multiplied
-// by sigmoid(gate) (the gate comes after). `rows`: out[r] is the norm of x[rows[r]] (the gate's rows are not gathered).
+// by sigmoid(gate) (the gate comes after); gate_kind 3: by silu(gate), also after. `rows`: out[r] is the norm of x[rows[r]] (the gate's rows are not gathered).
 template <typename TX, typename TG, typename TO>
 __global__ __launch_bounds__(1024) void group_rmsnorm_kernel(const TX* __restrict__ x, int ldx, const float* __restrict__ w,
                                                             TO* __restrict__ out, int ldo, const int* __restrict__ rows,
@@ -172,6 +172,7 @@ __global__ __launch_bounds__(1024) void group_rmsnorm_kernel(const TX* __restric
     auto finish = [&](int i, float v) {
         float y = v * inv * w[c0 + i];
         if (gate_kind == 2) y *= 1.0f / (1.0f + expf(-to_f32(gsrc[i])));
+        if (gate_kind == 3) { const float z = to_f32(gsrc[i]); y *= z / (1.0f + expf(-z)); }
         dst[i] = from_f32<TO>(y);
     };
 #pragma unroll
@@ -190,7 +191,7 @@ extern "C" int hfa_group_rmsnorm(const void* x, int x_dtype, int ldx, const floa
     HFA_REQUIRE(groups > 0 && width % groups == 0 && groups <= 65535, "group_rmsnorm: %d values do not form %d equal runs", width, groups);
     HFA_REQUIRE((x_dtype == HFA_F32 || x_dtype == HFA_BF16) && (out_dtype == HFA_F32 || out_dtype == HFA_BF16),
                 "group_rmsnorm: unknown dtype");
-    HFA_REQUIRE(gate_kind >= 0 && gate_kind <= 2 && (gate_kind == 0 || (gate && ldg >= width && !rows &&
+    HFA_REQUIRE(gate_kind >= 0 && gate_kind <= 3 && (gate_kind == 0 || (gate && ldg >= width && !rows &&
                                                                        (gate_dtype == HFA_F32 || gate_dtype == HFA_BF16))),
                 "group_rmsnorm: a gate needs its rows, one for each row in order");
     const int run = width / groups;
@@ -206,5 +207,59 @@ extern "C" int hfa_group_rmsnorm(const void* x, int x_dtype, int ldx, const floa
     else { if (gb) GRN(bf16, bf16, bf16); else GRN(bf16, float, bf16); }
 #undef GRN
     HFA_LAUNCH_CHECK("group_rmsnorm");
+    return 0;
+}
+
+// ---- a branch's result on its way into the stream, and a gate on a mixer's heads ---------------------
+// hfa_scale_add: out[r, c] (+)= scale * col[c] * y[r, c] in fp32 (col null: 1): a residual sum whose branch is multiplied by
+// one number and, column by column, by a learned vector.
+__global__ void scale_add_kernel(const float* __restrict__ y, int ldy, const float* __restrict__ col, float scale,
+                                 float* __restrict__ out, int ldo, int width, int accumulate, size_t total) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t r = i / width, c = i % width;
+        const float v = (col ? scale * col[c] : scale) * y[r * ldy + c];
+        float* o = out + r * ldo + c;
+        *o = accumulate ? *o + v : v;
+    }
+}
+
+extern "C" int hfa_scale_add(const float* y, int ldy, const float* col, float scale, float* out, int ldo, int n_rows, int width,
+                             int accumulate, hipStream_t stream) {
+    HFA_REQUIRE(y && out && n_rows > 0 && width > 0 && ldy >= width && ldo >= width, "scale_add: bad arguments");
+    const size_t total = (size_t)n_rows * width;
+    const int blocks = (int)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
+    scale_add_kernel<<<blocks, 256, 0, stream>>>(y, ldy, col, scale, out, ldo, width, accumulate, total);
+    HFA_LAUNCH_CHECK("scale_add");
+    return 0;
+}
+
+// hfa_gate_mul: out[r, c] = x[r, c] * act(gate[r, c]), the product formed in fp32 (act: HFA_ACT_SIGMOID or HFA_ACT_SILU).
+template <typename TX, typename TG, typename TO>
+__global__ void gate_mul_kernel(const TX* __restrict__ x, int ldx, const TG* __restrict__ gate, int ldg, TO* __restrict__ out,
+                                int ldo, int width, int act, size_t total) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t r = i / width, c = i % width;
+        out[r * ldo + c] = from_f32<TO>(to_f32(x[r * ldx + c]) * hfa_act_apply(act, to_f32(gate[r * ldg + c])));
+    }
+}
+
+extern "C" int hfa_gate_mul(const void* x, int x_dtype, int ldx, const void* gate, int gate_dtype, int ldg, void* out, int out_dtype,
+                            int ldo, int n_rows, int width, int act, hipStream_t stream) {
+    HFA_REQUIRE(x && gate && out && n_rows > 0 && width > 0 && ldx >= width && ldg >= width && ldo >= width, "gate_mul: bad arguments");
+    HFA_REQUIRE(act == HFA_ACT_SIGMOID || act == HFA_ACT_SILU, "gate_mul: the gate's function is the logistic function or silu");
+    HFA_REQUIRE((x_dtype == HFA_F32 || x_dtype == HFA_BF16) && (gate_dtype == HFA_F32 || gate_dtype == HFA_BF16) &&
+                    (out_dtype == HFA_F32 || out_dtype == HFA_BF16), "gate_mul: unknown dtype");
+    const size_t total = (size_t)n_rows * width;
+    const int blocks = (int)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
+#define GM(TX, TG, TO) gate_mul_kernel<TX, TG, TO><<<blocks, 256, 0, stream>>>((const TX*)x, ldx, (const TG*)gate, ldg, (TO*)out, ldo, width, act, total)
+    const bool xb = x_dtype == HFA_BF16, gb = gate_dtype == HFA_BF16, ob = out_dtype == HFA_BF16;
+    if (xb && gb && ob) GM(bf16, bf16, bf16);
+    else if (!xb && !gb && !ob) GM(float, float, float);
+    else if (!xb && gb && ob) GM(float, bf16, bf16);
+    else if (!xb && !gb && ob) GM(float, float, bf16);
+    else if (xb && !gb && ob) GM(bf16, float, bf16);
+    else { hfa_set_error("gate_mul: this mix of dtypes is not built"); return 1; }
+#undef GM
+    HFA_LAUNCH_CHECK("gate_mul");
     return 0;
 }

@@ -605,3 +605,205 @@ extern "C" int hfa_delta_scan(const float* q, int ldq, const float* k, int ldk, 
     HFA_LAUNCH_CHECK("delta_scan");
     return 0;
 }
+
+// ---- a decay per key channel -------------------------------------------------------------------------------------------
+// Per head, S [N][P] in the state row, in hfa_linear_scan's layout: S <- diag(a_t) S + k_t v_t^T, y_t = S^T (q_scale q_t). The
+// decays are formed here, in fp32, from z = gate[t, h N + n] + gate_bias[h N + n]:
+//   form 0: a = lower[h N + n] + (1 - lower[h N + n]) sigmoid(z), and the key is the decay's complement, k = 1 - a (a forget gate
+//           that also decides what is written; no keys are read);
+//   form 1: a = sigmoid(z)^inv_tau, as exp(inv_tau logsigmoid(z)); keys are read.
+// q_act HFA_ACT_SILU: the queries pass silu on their way in. The block, its lanes and the staging through LDS are
+// linear_scan_kernel's, with the decays staged beside the keys as delta_scan_kernel stages its own; nothing crosses lanes
+// inside the walk.
+template <typename T, typename TG, int NS, int NPT>
+__global__ __launch_bounds__(SCAN_THREADS) void channel_scan_kernel(
+    const T* __restrict__ q, int ldq, const T* __restrict__ k, int ldk, int N, const T* __restrict__ v, int ldv, int P,
+    const TG* __restrict__ gate, int ld_gate, const float* __restrict__ gate_bias, int form, const float* __restrict__ lower,
+    float inv_tau, int q_act, float q_scale, float* __restrict__ state, size_t state_ld, const int* __restrict__ q_start,
+    const int* __restrict__ seq_slot, float* __restrict__ y, int ldy) {
+    constexpr int NPAD = NS * NPT, PT = SCAN_THREADS / NS, TOK = SCAN_TOKENS;
+    constexpr int RK = TOK * NPAD / SCAN_THREADS, RV = (TOK * PT + SCAN_THREADS - 1) / SCAN_THREADS;
+    static_assert(TOK * NPAD % SCAN_THREADS == 0 && NPT % 4 == 0, "the staging loops are whole");
+    __shared__ __attribute__((aligned(16))) float k_s[TOK * NPAD];
+    __shared__ __attribute__((aligned(16))) float q_s[TOK * NPAD];
+    __shared__ __attribute__((aligned(16))) float g_s[TOK * NPAD];
+    __shared__ float v_s[TOK * PT];
+    __shared__ __attribute__((aligned(16))) float part_s[TOK * SCAN_THREADS];
+    const int h = blockIdx.x, s = blockIdx.y, pz = blockIdx.z, tid = threadIdx.x;
+    const int pl = tid / NS, ns = tid % NS;
+    const int q0 = q_start[s], n_tok = q_start[s + 1] - q0;
+    if (n_tok <= 0) return;
+    const int p_pad = (int)gridDim.z * PT;
+    float* S = state + (size_t)seq_slot[s] * state_ld + (size_t)h * NPT * p_pad * NS + (size_t)pz * SCAN_THREADS + tid;
+    float st[NPT];
+#pragma unroll
+    for (int i = 0; i < NPT; i++) st[i] = S[(size_t)i * p_pad * NS];
+    const T* kg = k ? k + (size_t)q0 * ldk + h * N : nullptr;
+    const T* qg = q + (size_t)q0 * ldq + h * N;
+    const TG* gg = gate + (size_t)q0 * ld_gate + h * N;
+    const T* vg = v + (size_t)q0 * ldv + h * P + pz * PT;
+    float bias_r[RK], lower_r[RK];                         // of the channels this thread stages
+#pragma unroll
+    for (int r = 0; r < RK; r++) {
+        const int n = (tid + r * SCAN_THREADS) % NPAD;
+        bias_r[r] = (n < N && gate_bias) ? gate_bias[h * N + n] : 0.f;
+        lower_r[r] = (n < N && form == 0) ? lower[h * N + n] : 0.f;
+    }
+    struct Staged { float k[RK], q[RK], z[RK], v[RV]; };
+    Staged set_a, set_b;
+    auto fetch = [&](Staged& g_, int c0) {
+        if (c0 >= n_tok) return;
+#pragma unroll
+        for (int r = 0; r < RK; r++) {
+            const int idx = tid + r * SCAN_THREADS, t = c0 + idx / NPAD, n = idx % NPAD;
+            const bool ok = t < n_tok && n < N;
+            g_.k[r] = (ok && form == 1) ? to_f32(kg[(size_t)t * ldk + n]) : 0.f;
+            g_.q[r] = ok ? to_f32(qg[(size_t)t * ldq + n]) : 0.f;
+            g_.z[r] = ok ? to_f32(gg[(size_t)t * ld_gate + n]) : 0.f;
+        }
+#pragma unroll
+        for (int r = 0; r < RV; r++) {
+            const int idx = tid + r * SCAN_THREADS, t = c0 + idx / PT, pp = idx % PT;
+            g_.v[r] = (idx < TOK * PT && t < n_tok && pz * PT + pp < P) ? to_f32(vg[(size_t)t * ldv + pp]) : 0.f;
+        }
+    };
+    auto stash = [&](const Staged& g_) {
+#pragma unroll
+        for (int r = 0; r < RK; r++) {
+            const int idx = tid + r * SCAN_THREADS, n = idx % NPAD;
+            const float z = g_.z[r] + bias_r[r];
+            float a, kk;
+            if (form == 0) {
+                a = lower_r[r] + (1.0f - lower_r[r]) * (1.0f / (1.0f + expf(-z)));
+                kk = 1.0f - a;
+            } else {
+                const float ls = -(fmaxf(-z, 0.f) + log1pf(expf(-fabsf(z))));       // logsigmoid, exact for every z
+                a = expf(inv_tau * ls);
+                kk = g_.k[r];
+            }
+            const bool live = n < N;                       // rows beyond N stay zero
+            g_s[idx] = live ? a : 0.f;
+            k_s[idx] = live ? kk : 0.f;
+            const float qv = g_.q[r];
+            q_s[idx] = (q_act == HFA_ACT_SILU ? qv / (1.0f + expf(-qv)) : qv) * q_scale;
+        }
+#pragma unroll
+        for (int r = 0; r < RV; r++)
+            if (tid + r * SCAN_THREADS < TOK * PT) v_s[tid + r * SCAN_THREADS] = g_.v[r];
+    };
+    auto chunk = [&](Staged& g_, int c0) {
+        const int nt = n_tok - c0 < TOK ? n_tok - c0 : TOK;
+        __syncthreads();                                   // the walk before has read what is overwritten now
+        stash(g_);
+        __syncthreads();
+        fetch(g_, c0 + 2 * TOK);
+        struct Operands { float4 k[NPT / 4], q[NPT / 4], g[NPT / 4]; float v; };
+        auto read = [&](int t, Operands& o) {
+            const float4* kt = reinterpret_cast<const float4*>(k_s + t * NPAD + ns * NPT);
+            const float4* qt = reinterpret_cast<const float4*>(q_s + t * NPAD + ns * NPT);
+            const float4* gt = reinterpret_cast<const float4*>(g_s + t * NPAD + ns * NPT);
+#pragma unroll
+            for (int i = 0; i < NPT / 4; i++) {
+                o.k[i] = kt[i];
+                o.q[i] = qt[i];
+                o.g[i] = gt[i];
+            }
+            o.v = v_s[t * PT + pl];
+        };
+        auto token = [&](int t, const Operands& o) {
+            float acc0 = 0.f, acc1 = 0.f;
+#pragma unroll
+            for (int i = 0; i < NPT / 4; i++) {
+                const float4 a4 = o.g[i], kk = o.k[i], qq = o.q[i];
+                st[4 * i] = fmaf(a4.x, st[4 * i], kk.x * o.v);
+                st[4 * i + 1] = fmaf(a4.y, st[4 * i + 1], kk.y * o.v);
+                st[4 * i + 2] = fmaf(a4.z, st[4 * i + 2], kk.z * o.v);
+                st[4 * i + 3] = fmaf(a4.w, st[4 * i + 3], kk.w * o.v);
+                acc0 = fmaf(st[4 * i], qq.x, acc0);
+                acc1 = fmaf(st[4 * i + 1], qq.y, acc1);
+                acc0 = fmaf(st[4 * i + 2], qq.z, acc0);
+                acc1 = fmaf(st[4 * i + 3], qq.w, acc1);
+            }
+            part_s[t * SCAN_THREADS + tid] = acc0 + acc1;
+        };
+        if (nt == TOK) {
+            Operands ring[3];
+            read(0, ring[0]);
+            read(1, ring[1]);
+#pragma unroll
+            for (int t = 0; t < TOK; t++) {
+                if (t + 2 < TOK) read(t + 2, ring[(t + 2) % 3]);
+                token(t, ring[t % 3]);
+            }
+        } else {
+            for (int t = 0; t < nt; t++) {
+                Operands o;
+                read(t, o);
+                token(t, o);
+            }
+        }
+        __syncthreads();
+        for (int idx = tid; idx < nt * PT; idx += SCAN_THREADS) {
+            const int t = idx / PT, pp = idx % PT;
+            if (pz * PT + pp >= P) continue;
+            const float4* sh = reinterpret_cast<const float4*>(part_s + t * SCAN_THREADS + pp * NS);
+            float acc = 0.f;
+#pragma unroll
+            for (int i = 0; i < NS / 4; i++) {
+                const float4 w4 = sh[i];
+                acc = ((acc + w4.x) + w4.y) + w4.z + w4.w;
+            }
+            y[(size_t)(q0 + c0 + t) * ldy + h * P + pz * PT + pp] = acc;
+        }
+    };
+    fetch(set_a, 0);
+    fetch(set_b, TOK);
+    for (int c0 = 0; c0 < n_tok; c0 += 2 * TOK) {
+        chunk(set_a, c0);
+        if (c0 + TOK < n_tok) chunk(set_b, c0 + TOK);
+    }
+#pragma unroll
+    for (int i = 0; i < NPT; i++) S[(size_t)i * p_pad * NS] = st[i];
+}
+
+extern "C" int hfa_channel_scan(const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, int dtype, const void* gate,
+                                int gate_dtype, int ld_gate, const float* gate_bias, int form, const float* lower, float inv_tau,
+                                int q_act, int n_heads, int qk_dim, int v_dim, float q_scale, float* state, size_t state_ld,
+                                const int* q_start, const int* seq_slot, int n_seqs, float* y, int ldy, hipStream_t stream) {
+    HFA_REQUIRE(q && v && gate && state && q_start && seq_slot && y && n_seqs > 0, "channel_scan: a null argument");
+    HFA_REQUIRE(n_heads > 0 && qk_dim > 0 && v_dim > 0, "channel_scan: bad sizes");
+    HFA_REQUIRE((form == 0 && lower) || (form == 1 && k && inv_tau > 0.f),
+                "channel_scan: form 0 needs the decays' lower bounds, form 1 keys and a positive 1 / tau");
+    HFA_REQUIRE(q_act == HFA_ACT_NONE || q_act == HFA_ACT_SILU, "channel_scan: the queries pass silu or nothing");
+    HFA_REQUIRE(qk_dim <= 256, "channel_scan: a state of %d rows a head is too large (at most 256)", qk_dim);
+    HFA_REQUIRE(ldq >= n_heads * qk_dim && (form == 0 || ldk >= n_heads * qk_dim) && ldv >= n_heads * v_dim && ldy >= n_heads * v_dim &&
+                    ld_gate >= n_heads * qk_dim && state_ld >= hfa_linear_scan_state_floats(n_heads, qk_dim, v_dim),
+                "channel_scan: a row is shorter than its heads (a state row holds hfa_linear_scan_state_floats values)");
+    HFA_REQUIRE((dtype == HFA_F32 || dtype == HFA_BF16) && (gate_dtype == HFA_F32 || gate_dtype == HFA_BF16) &&
+                    !(dtype == HFA_F32 && gate_dtype == HFA_BF16), "channel_scan: unknown mix of dtypes");
+    int ns, npt;
+    scan_shape(qk_dim, &ns, &npt);
+    const int pt = SCAN_THREADS / ns, p_tiles = (v_dim + pt - 1) / pt;
+    HFA_REQUIRE(n_heads <= 65535 && n_seqs <= 65535 && p_tiles <= 65535, "channel_scan: the step exceeds the grid");
+    dim3 grid(n_heads, n_seqs, p_tiles);
+#define CH_GO(T, TG, NS, NPT)                                                                                              \
+    channel_scan_kernel<T, TG, NS, NPT><<<grid, SCAN_THREADS, 0, stream>>>(                                                \
+        (const T*)q, ldq, (const T*)k, ldk, qk_dim, (const T*)v, ldv, v_dim, (const TG*)gate, ld_gate, gate_bias, form, lower, \
+        inv_tau, q_act, q_scale, state, state_ld, q_start, seq_slot, y, ldy)
+#define CH_SIZES(T, TG)                                          \
+    do {                                                         \
+        if (ns == 4) CH_GO(T, TG, 4, 4);                         \
+        else if (ns == 8 && npt == 4) CH_GO(T, TG, 8, 4);        \
+        else if (ns == 8) CH_GO(T, TG, 8, 8);                    \
+        else if (npt == 4) CH_GO(T, TG, 16, 4);                  \
+        else if (npt == 8) CH_GO(T, TG, 16, 8);                  \
+        else CH_GO(T, TG, 16, 16);                               \
+    } while (0)
+    if (dtype == HFA_F32) CH_SIZES(float, float);
+    else if (gate_dtype == HFA_F32) CH_SIZES(bf16, float);
+    else CH_SIZES(bf16, bf16);
+#undef CH_SIZES
+#undef CH_GO
+    HFA_LAUNCH_CHECK("channel_scan");
+    return 0;
+}

@@ -621,7 +621,7 @@ class Ops:
             None if pend is None or pend.bias is None else pend.bias.data_ptr(), self._stream()))
 
     def paged_attention(self, q, n_heads, n_kv_heads, head_dim, cache, step, window, scale, out, slopes=None,
-                        v_head_dim=None, mask_chunk=0, sink=False, cross_values=False):
+                        v_head_dim=None, mask_chunk=0, sink=False, cross_values=False, softcap=0.0, weights="softmax", head_bias=None):
         """Attention of the first ``n_heads * head_dim`` columns of ``q`` over ``cache``. ``slopes``
         (fp32, one per query head): the score of key j for the query at p gets ``slopes[h] * (j - p)``
         added, for position encodings that enter the scores; the plain kernel then runs, as it does when
@@ -630,13 +630,22 @@ class Ops:
         ``sink``: the softmax's denominator holds one more term of score 0 that has no value. ``cross_values``: every
         head's weights are applied to the values of every key/value group; ``out`` is ``[T, groups * heads * v_head_dim]``,
         round r of head h (at ``(r * heads + h) * v_head_dim``) being its weights on the values of group (h's group + r) mod
-        groups (see ``talk_mix``)."""
+        groups (see ``talk_mix``). ``softcap`` c > 0: a score becomes ``c tanh(score / c)`` before the weights are formed.
+        ``weights`` ``"sigmoid"``: no softmax; a visible key weighs ``sigmoid(score + head_bias[h])`` (``head_bias``: fp32, one per
+        query head, or None), and the weights are not normalised over the keys. Both take the plain kernel."""
         v_head_dim = head_dim if v_head_dim is None else int(v_head_dim)
         mask_chunk = int(mask_chunk)
+        if weights not in ("softmax", "sigmoid") or (weights == "sigmoid" and (sink or cross_values)):
+            fail(ENOTSUP, f"paged_attention: weights '{weights}' are softmax or sigmoid (the latter without a sink term or mixed heads)")
+        if head_bias is not None and (weights != "sigmoid" or head_bias.dtype != torch.float32 or head_bias.numel() != n_heads
+                                      or not head_bias.is_contiguous() or head_bias.device != q.device):
+            fail(EINVAL, "paged_attention: head_bias goes with sigmoid weights and is contiguous fp32 on the device, one per query head")
+        softcap = float(softcap or 0.0)
+        shaped_scores = softcap != 0.0 or weights != "softmax"
         self._scaled.pop(out.data_ptr(), None)               # whatever `out` held, it is no norm's lazy output any more
         lr = self._lazy_rope
         if lr is not None and lr.qkv.data_ptr() == q.data_ptr() and lr.cache is cache and slopes is None and not sink \
-                and not cross_values \
+                and not cross_values and not shaped_scores \
                 and step.max_q_len == 1 and step.n_seqs == q.shape[0] and not self.force_plain_attention \
                 and out.dtype == torch.bfloat16 and v_head_dim == head_dim and lr.args[4] == n_heads and lr.args[6] == head_dim \
                 and lr.args[5] in (0, n_kv_heads) and cache.k.shape[1] == n_kv_heads * head_dim \
@@ -674,7 +683,8 @@ class Ops:
                 step.token_slot.data_ptr() + 4 * first, step.positions.data_ptr() + 4 * first, q_start.data_ptr(), n_seqs,
                 max_q_len, step.max_seq_len, out.data_ptr() + first * ldo * out.element_size(), ldo, n_tokens, n_heads,
                 n_kv_heads, head_dim, v_head_dim, cache.page_tokens, int(window), mask_chunk, float(scale),
-                None if slopes is None else slopes.data_ptr(), 1 if sink else 0, 1 if cross_values else 0, self.attn_workspace.data_ptr(),
+                None if slopes is None else slopes.data_ptr(), 1 if sink else 0, 1 if cross_values else 0, softcap,
+                1 if weights == "sigmoid" else 0, None if head_bias is None else head_bias.data_ptr(), self.attn_workspace.data_ptr(),
                 self.attn_workspace.numel(), 1 if plain else 0, self._stream()))
 
         # Decoded tokens beside prompt portions: one call would send all of them to the kernel for prompt
@@ -682,7 +692,8 @@ class Ops:
         # take as long as thousands of prompt tokens). The step lays requests with few tokens first, so
         # each part is a step of its own: the first goes to the kernel that cuts the keys into chunks.
         n_short = getattr(step, "n_short_seqs", 0)
-        if not plain and q.dtype == torch.bfloat16 and step.max_q_len >= self.prompt_rows and 0 < n_short < step.n_seqs:
+        if not plain and not shaped_scores and v_head_dim == head_dim and q.dtype == torch.bfloat16 \
+                and step.max_q_len >= self.prompt_rows and 0 < n_short < step.n_seqs:
             ts = step.n_short_tokens
             _ints(step.q_start_long, "q_start_long", step.n_seqs - n_short + 1)
             call(0, ts, step.q_start, n_short, step.max_short_q_len)
@@ -727,13 +738,13 @@ class Ops:
         self._check(self.lib.hfa_swiglu(gate_up.data_ptr(), out.data_ptr(), _code(out), T, F2 // 2, self._stream()))
 
     # ---- norms in groups, queries and keys normed whole, mixers with per-request state -------------------------------
-    GATES = {None: 0, "silu_before": 1, "sigmoid_after": 2}
+    GATES = {None: 0, "silu_before": 1, "sigmoid_after": 2, "silu_after": 3}
 
     def group_rmsnorm(self, x, weight, eps, groups, out, rows=None, gate=None, gate_kind=None, row_scale=None):
         """``out[r] = norm(x[rows[r]])``: the row is cut into ``groups`` equal runs, each divided by its own root mean
         square (``eps`` inside the root), the whole times ``weight``; sums in fp32. ``gate`` (a matrix with the rows of
-        ``out``) with ``gate_kind`` ``silu_before`` (the row times silu(gate) is normed) or ``sigmoid_after`` (the normed
-        row is multiplied by sigmoid(gate)). ``row_scale`` (fp32 [rows, groups]): run g of row r is multiplied by
+        ``out``) with ``gate_kind`` ``silu_before`` (the row times silu(gate) is normed), ``sigmoid_after`` (the normed
+        row is multiplied by sigmoid(gate)) or ``silu_after`` (by silu(gate)). ``row_scale`` (fp32 [rows, groups]): run g of row r is multiplied by
         ``row_scale[r, g]`` before everything else (a recurrence's denominator, a head at a time)."""
         self.settle()
         self._whole(x)
@@ -906,6 +917,84 @@ class Ops:
             float(q_scale), float(unit_eps), state.data_ptr(), state.stride(0), _ints(step.q_start, "q_start", step.n_seqs + 1),
             _ints(step.seq_slot, "seq_slot", step.n_seqs), step.n_seqs, int(step.max_q_len), y.data_ptr(), _rows(y, "scan out"), self._stream()))
 
+    def channel_scan(self, q, k, v, n_heads, qk_dim, v_dim, gate, gate_bias, state, step, y, lower=None, tau=None, q_act=None,
+                     q_scale=1.0):
+        """A recurrence with a decay per key channel, along each request's tokens from its row of ``state`` (fp32,
+        ``scan_state_floats`` values in ``linear_scan``'s order): ``S <- diag(a_t) S + k_t v_t^T``, ``y_t = S^T (q_scale q_t)`` (fp32).
+        The decays are formed in fp32 from ``z = gate[t] + gate_bias`` ([T, heads * qk_dim], the bias fp32 or None). With ``lower``
+        (fp32 [heads * qk_dim]): ``a = lower + (1 - lower) sigmoid(z)`` and ``k_t = 1 - a_t`` (``k`` is None: the forget gate decides
+        what is written). With ``tau``: ``a = sigmoid(z)^(1 / tau)``, keys from ``k``. ``q_act`` ``"silu"``: the queries pass silu first."""
+        self.settle()
+        for t in (q, k, v, gate):
+            if t is not None:
+                self._whole(t)
+        T = y.shape[0]
+        form = 0 if lower is not None else 1
+        if (lower is None) == (tau is None) or (form == 1) != (k is not None):
+            fail(EINVAL, "channel_scan: either lower bounds and no keys, or tau and keys")
+        if q.dtype != v.dtype or (k is not None and k.dtype != q.dtype) or y.dtype != torch.float32 or state.dtype != torch.float32 \
+                or state.stride(1) != 1 or q.shape[0] != T or v.shape[0] != T or gate.shape[0] != T or y.shape[1] != n_heads * v_dim \
+                or (q.dtype == torch.float32 and gate.dtype != torch.float32):
+            fail(EINVAL, "channel_scan: q, k and v of one dtype and the step's rows, fp32 output and state")
+        for t, what in ((gate_bias, "gate_bias"), (lower, "lower")):
+            if t is not None and (t.dtype != torch.float32 or t.numel() != n_heads * qk_dim or not t.is_contiguous()):
+                fail(EINVAL, f"channel_scan: {what} must be one fp32 value a (head, key channel)")
+        if state.shape[1] < self.scan_state_floats(n_heads, qk_dim, v_dim) or qk_dim > 256:
+            fail(EINVAL, f"channel_scan: a state row of {state.shape[1]} values for {n_heads} states of {qk_dim} x {v_dim} (at most 256 rows)")
+        if q_act not in (None, "silu"):
+            fail(ENOTSUP, f"channel_scan: the queries pass silu or nothing, not '{q_act}'")
+
+        def ptr(t):
+            return None if t is None else t.data_ptr()
+        self._check(self.lib.hfa_channel_scan(
+            q.data_ptr(), _rows(q, "scan q"), ptr(k), 0 if k is None else _rows(k, "scan k"), v.data_ptr(), _rows(v, "scan v"), _code(q),
+            gate.data_ptr(), _code(gate), _rows(gate, "scan gate"), ptr(gate_bias), form, ptr(lower), 0.0 if tau is None else 1.0 / float(tau),
+            self.ACTIVATIONS["silu"] if q_act else 0, n_heads, qk_dim, v_dim, float(q_scale), state.data_ptr(), state.stride(0),
+            _ints(step.q_start, "q_start", step.n_seqs + 1), _ints(step.seq_slot, "seq_slot", step.n_seqs), step.n_seqs, y.data_ptr(),
+            _rows(y, "scan out"), self._stream()))
+
+    def scale_add(self, y, out, scale=1.0, columns=None, accumulate=True):
+        """``out (+)= scale * columns * y`` in fp32, ``columns`` an fp32 vector with one factor a column (None: 1): a branch's
+        result on its way into the stream."""
+        self.settle()
+        self._source_changes(out)
+        self._scaled.pop(out.data_ptr(), None)
+        R, E = y.shape
+        if y.dtype != torch.float32 or out.dtype != torch.float32 or tuple(out.shape) != (R, E) \
+                or (columns is not None and (columns.dtype != torch.float32 or columns.numel() != E or not columns.is_contiguous())):
+            fail(EINVAL, "scale_add: y, out and the columns' factors must be fp32 and of one width")
+        self._check(self.lib.hfa_scale_add(y.data_ptr(), _rows(y, "scale_add in"), None if columns is None else columns.data_ptr(),
+                                           float(scale), out.data_ptr(), _rows(out, "scale_add out"), R, E, 1 if accumulate else 0,
+                                           self._stream()))
+
+    def gate_mul(self, x, gate, out, kind="sigmoid"):
+        """``out = x * act(gate)`` element by element, formed in fp32; ``kind`` is ``sigmoid`` or ``silu``. ``out`` may be ``x``."""
+        self.settle()
+        self._whole(x)
+        self._whole(gate)
+        self._scaled.pop(out.data_ptr(), None)
+        if kind not in ("sigmoid", "silu") or x.shape != gate.shape or x.shape != out.shape or x.dim() != 2:
+            fail(EINVAL, "gate_mul: x, gate and out of one shape; the gate's function is sigmoid or silu")
+        self._check(self.lib.hfa_gate_mul(x.data_ptr(), _code(x), _rows(x, "gate_mul x"), gate.data_ptr(), _code(gate), _rows(gate, "gate"),
+                                          out.data_ptr(), _code(out), _rows(out, "gate_mul out"), x.shape[0], x.shape[1],
+                                          self.ACTIVATIONS[kind], self._stream()))
+
+    def latent_pack(self, down, q, weight, eps, packed, n_heads, dim, rot, latent):
+        """The rows that ``rope_store`` and ``paged_attention`` take for attention through latents with one key/value head
+        (key ``[rotated part | latent]``, value the latent): from ``down`` (fp32 [T, latent + rot]: the latent before its norm, then
+        the key's part to be rotated) and ``q`` ([T, heads * (dim + rot)], a head being ``[dim | rot]``) it writes
+        ``packed[t] = [heads x (rot | latent: left alone) | rot | latent | latent]``, the latent RMS-normed with ``weight``."""
+        self.settle()
+        self._whole(q)
+        T = down.shape[0]
+        if down.dtype != torch.float32 or down.shape[1] < latent + rot or q.shape[0] != T or q.shape[1] < n_heads * (dim + rot) \
+                or packed.shape[0] != T or packed.shape[1] < n_heads * (rot + latent) + rot + 2 * latent \
+                or weight.dtype != torch.float32 or weight.numel() != latent or not weight.is_contiguous():
+            fail(EINVAL, "latent_pack: rows of the latent and the rotated part (fp32), the heads' queries, an fp32 weight of the latent's size")
+        self._check(self.lib.hfa_latent_pack(down.data_ptr(), _rows(down, "latent rows"), q.data_ptr(), _code(q), _rows(q, "queries"),
+                                             weight.data_ptr(), float(eps), packed.data_ptr(), _code(packed), _rows(packed, "packed rows"),
+                                             T, n_heads, dim, rot, latent, self._stream()))
+
     # ---- layer norm, plain activations, soft cap -----------------------------------------------------------------
     def layernorm(self, x, weight, bias, eps, out, rows=None):
         """``out[r] = (x[rows[r]] - mean) / sqrt(var + eps) * weight + bias`` in fp32 (``bias`` None: no shift). A
@@ -952,20 +1041,24 @@ class Ops:
             self._check(self.lib.hfa_softcap(x.data_ptr(), _rows(x, "softcap"), x.shape[0], x.shape[1], float(cap), self._stream()))
 
     # ---- mixture of experts ------------------------------------------------------------------------------------------
+    SCORINGS = {"softmax": 0, "sigmoid": 1, "softmax_chosen": 2}
+
     def moe_route(self, logits, top, n_groups, keep, scoring="softmax", renorm=True, out_scale=1.0):
-        """(ids [T, top] int32, weights [T, top] fp32) from fp32 router logits [T, E]: see ``hfa_moe_route``."""
+        """(ids [T, top] int32, weights [T, top] fp32) from fp32 router logits [T, E]: see ``hfa_moe_route``. ``scoring``
+        ``softmax_chosen``: the experts with the largest logits, weighted (with ``renorm``) by the softmax over the chosen
+        logits alone."""
         self.settle()
         T, E = logits.shape
-        if logits.dtype != torch.float32 or scoring not in ("softmax", "sigmoid"):
-            fail(EINVAL, "moe_route: fp32 logits and softmax or sigmoid scoring")
+        if logits.dtype != torch.float32 or scoring not in self.SCORINGS:
+            fail(EINVAL, f"moe_route: fp32 logits and a scoring among {', '.join(self.SCORINGS)}")
         ids = self.scratch("moe_ids", (T, top), torch.int32)
         wts = self.scratch("moe_weights", (T, top), torch.float32)
         self._check(self.lib.hfa_moe_route(logits.data_ptr(), _rows(logits, "router logits"), T, E, int(top), int(n_groups), int(keep),
-                                           0 if scoring == "softmax" else 1, 1 if renorm else 0, float(out_scale),
+                                           self.SCORINGS[scoring], 1 if renorm else 0, float(out_scale),
                                            ids.data_ptr(), wts.data_ptr(), self._stream()))
         return ids, wts
 
-    def moe_experts(self, h, ids, weights, w_up, w_down, act, x, gated=None):
+    def moe_experts(self, h, ids, weights, w_up, w_down, act, x, gated=None, weight_on="input"):
         """``x[t] += sum_k weights[t, k] * w_down[ids[t, k]] act(w_up[ids[t, k]] h[t])``: ``w_up`` is [E, F, width],
         ``w_down`` [E, width, F]. The pairs are put in expert order on the device, each expert's rows go through the
         two products in tiles, and the weighted results are added to ``x`` (fp32) choice by choice.
@@ -975,7 +1068,9 @@ class Ops:
         32 gate rows and 32 up rows (``interleave_experts``); with ``c = weights[t, k]``, ``g = min(c Wgate h, limit)``, ``u =
         clamp(c Wup h, -limit, limit)`` (``limit`` <= 0: unbounded) the expert gives ``Wdown (g sigmoid(alpha g) (u + shift))``,
         unweighted; ``act`` is ignored. Interleaved, the up product's last lines form the activation from its 32-bit sums;
-        otherwise the sums pass through memory and a kernel of its own forms it."""
+        otherwise the sums pass through memory and a kernel of its own forms it. ``weight_on`` ``"output"`` (gated experts only;
+        experts without a gate always weigh their output): c = 1 inside the expert, and the down product's rows are multiplied
+        by the pair's weight instead."""
         self.settle()
         self._whole(h)
         self._source_changes(x)
@@ -1009,6 +1104,7 @@ class Ops:
         y = self.scratch("moe_out", (n_pairs, W), torch.float32)
         if gated is not None:
             alpha, limit, shift, interleaved = gated
+            w_in, w_out = (weights, None) if weight_on == "input" else (None, weights)
             # A row or two an expert (a few decoded tokens): the experts' matrices are streamed once, by blocks that own 32 of
             # their rows each; blocks that own a gate block and its up block are half as many and stream slower (835 against
             # 900 us for the experts of a step of 8 tokens, 64 experts of 1,024 x 4,096; at 64 tokens 1,440 against 1,395),
@@ -1017,13 +1113,14 @@ class Ops:
             if interleaved and not streamed:
                 self._check(self.lib.hfa_moe_gemm(h.data_ptr(), _rows(h, "moe h"), code, top, w_up.data_ptr(), wcode, row_pair.data_ptr(),
                                                   tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, tile_rows, mid.data_ptr(), F, code, 0,
-                                                  weights.data_ptr(), 0, F_up, W, plain, 1, float(alpha), float(limit), float(shift),
-                                                  self._stream()))
+                                                  None if w_in is None else w_in.data_ptr(), 0, F_up, W, plain, 1, float(alpha),
+                                                  float(limit), float(shift), self._stream()))
             else:
-                self._gated_in_two(h, code, top, w_up, wcode, row_pair, tiles, n_tiles, max_tiles, tile_rows, mid, weights, n_pairs,
+                self._gated_in_two(h, code, top, w_up, wcode, row_pair, tiles, n_tiles, max_tiles, tile_rows, mid, w_in, n_pairs,
                                    F, F_up, W, plain, alpha, limit, shift, interleaved)
             self._check(self.lib.hfa_moe_gemm(mid.data_ptr(), F, code, 0, w_down.data_ptr(), wcode, row_pair.data_ptr(), tiles.data_ptr(),
-                                              n_tiles.data_ptr(), max_tiles, tile_rows, y.data_ptr(), W, F32, 1, None, 0, W, F,
+                                              n_tiles.data_ptr(), max_tiles, tile_rows, y.data_ptr(), W, F32, 1,
+                                              None if w_out is None else w_out.data_ptr(), 0, W, F,
                                               plain, 0, 0.0, 0.0, 0.0, self._stream()))
             self._check(self.lib.hfa_moe_combine(y.data_ptr(), x.data_ptr(), T, top, W, self._stream()))
             return
@@ -1037,7 +1134,8 @@ class Ops:
         self._check(self.lib.hfa_moe_gemm(h.data_ptr(), _rows(h, "moe h"), code, top, w_up.data_ptr(), wcode, row_pair.data_ptr(),
                                           tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, tile_rows, sums.data_ptr(), F_up, F32, 0,
                                           None, 0, F_up, W, plain, 0, 0.0, 0.0, 0.0, self._stream()))
-        self._check(self.lib.hfa_moe_gated_act(sums.data_ptr(), F_up, row_pair.data_ptr(), weights.data_ptr(), mid.data_ptr(), code, F,
+        self._check(self.lib.hfa_moe_gated_act(sums.data_ptr(), F_up, row_pair.data_ptr(), None if weights is None else weights.data_ptr(),
+                                               mid.data_ptr(), code, F,
                                                n_pairs, F, float(alpha), float(limit), float(shift), 1 if interleaved else 0,
                                                self._stream()))
 

@@ -1,2 +1,2 @@
 """Architectures. Importing this package registers them."""
-from . import qwen2, goridra, tobozen, mobupel   # noqa: F401
+from . import qwen2, goridra, tobozen, mobupel, gitasun   # noqa: F401

@@ -8,16 +8,59 @@ from .base import ParamSpec, Part
 @register_part("block", "prenorm")
 class PreNormBlock(Part):
     """``x += mixer(norm1(x)); x += feed_forward(norm2(x))`` (src/model.c:580-623):
-    norms in front of each part, nothing after, the residual stream in fp32."""
+    norms in front of each part, nothing after, the residual stream in fp32.
+
+    ``branch_scale`` m and ``layer_scales`` = {"mixer": name, "feed_forward": name} (tensors of the model's width, after
+    ``prefix``): a branch's result is multiplied by m and, element by element, by its vector before it joins the stream,
+    ``x += m * ls * branch(norm(x))``. The branch's result, the factors and the sum are fp32: the branch is computed into a
+    buffer of its own and added by one kernel."""
     graph_safe = True
 
 
-    def __init__(self, hidden_size, prefix=""):
+    def __init__(self, hidden_size, prefix="", branch_scale=None, layer_scales=None):
         super().__init__(prefix)
         self.E = hidden_size
+        self.branch_scale = None if branch_scale is None else float(branch_scale)
+        self.scale_names = dict(layer_scales or {})
+        self.scales = {}
+
+    def param_specs(self):
+        return [ParamSpec(self.prefix + n, (self.E,), "vector", ("one_plus_normal", 0.1)) for n in self.scale_names.values()]
+
+    def bind(self, params, ops):
+        self.scales = {k: params[self.prefix + n].contiguous() for k, n in self.scale_names.items()}
+
+    def _scaled_branch(self, ops, x, which, part, run):
+        """``x += branch_scale * layer_scale[which] * branch``; ``run(y, overwrite)`` makes the part write (or add) its result into ``y``."""
+        y = ops.scratch("branch", (x.shape[0], self.E), torch.float32)
+        if getattr(part, "can_overwrite", False):
+            run(y, True)
+        else:                                  # a part that only knows how to add: into zeros
+            ops.settle()
+            y.zero_()
+            run(y, False)
+        with ops.section("branch_sum"):
+            ops.scale_add(y, x, scale=1.0 if self.branch_scale is None else self.branch_scale, columns=self.scales.get(which))
+
+    def _forward_scaled(self, ops, step, x, parts, caches, write_cache):
+        h = ops.scratch("normed", (x.shape[0], self.E), ops.act_dtype)
+        parts["norm1"].forward(ops, x, h)
+        ops.settle(x)
+        mixer, cache = parts["mixer"], caches.get("mixer")
+        self._scaled_branch(ops, x, "mixer", mixer, lambda y, over: mixer.forward(ops, step, h, cache, y, write_cache, accumulate=False)
+                            if over else mixer.forward(ops, step, h, cache, y, write_cache))
+        ff = parts.get("feed_forward")
+        if ff is None:
+            return
+        parts["norm2"].forward(ops, x, h)
+        ops.settle(x)
+        self._scaled_branch(ops, x, "feed_forward", ff, lambda y, over: ff.forward(ops, step, h, y, accumulate=False)
+                            if over else ff.forward(ops, step, h, y))
 
     def forward(self, ops, step, x, parts, caches, write_cache=True):
         """``parts``: norm1, mixer, norm2, feed_forward; ``caches``: the mixer's, under its name."""
+        if self.branch_scale is not None or self.scale_names:
+            return self._forward_scaled(ops, step, x, parts, caches, write_cache)
         h = ops.scratch("normed", (x.shape[0], self.E), ops.act_dtype)
         norm_for(ops, parts["norm1"], parts["mixer"], x, h)      # also adds up a product the previous part deferred into x
         ops.settle(x)                          # (nothing left to do unless the norm could not)

@@ -12,28 +12,30 @@ from .base import ParamSpec, Part
 class GatedMLP(Part):
     """``x += Wdown (act(Wgate h) * (Wup h))`` with ``act(g) = g / (1 + exp(-g))``
     (src/model.c:612-623, src/mathx.c:34). Gate and up share their input and are held
-    as one matrix, gate rows first."""
+    as one matrix, gate rows first. ``names``: the tensors' names after ``prefix`` (keys gate, up, down)."""
     graph_safe = True
     lazy_input_ok = True
 
 
-    def __init__(self, hidden_size, intermediate_size, activation="silu", prefix=""):
+    def __init__(self, hidden_size, intermediate_size, activation="silu", prefix="", names=None):
         super().__init__(prefix)
         if activation != "silu":
             fail(ENOTSUP, f"gated_mlp: activation '{activation}' is not implemented")
         self.E, self.F = hidden_size, intermediate_size
+        self.names = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
+        self.names.update(names or {})
         self.w_gate_up = self.w_down = None
         self.fused = False
 
     def param_specs(self):
-        p = self.prefix
-        return [ParamSpec(p + "gate_proj.weight", (self.F, self.E)),
-                ParamSpec(p + "up_proj.weight", (self.F, self.E)),
-                ParamSpec(p + "down_proj.weight", (self.E, self.F))]
+        p, nm = self.prefix, self.names
+        return [ParamSpec(p + nm["gate"], (self.F, self.E)),
+                ParamSpec(p + nm["up"], (self.F, self.E)),
+                ParamSpec(p + nm["down"], (self.E, self.F))]
 
     def bind(self, params, ops):
-        p = self.prefix
-        g, u = params[p + "gate_proj.weight"], params[p + "up_proj.weight"]
+        p, nm = self.prefix, self.names
+        g, u = params[p + nm["gate"]], params[p + nm["up"]]
         dt = torch.float32 if torch.float32 in (g.dtype, u.dtype) else g.dtype
         # On the matrix cores gate and up rows are interleaved in blocks of 32, so that the product's
         # last step can form silu(gate) * up without storing gate and up.
@@ -43,7 +45,7 @@ class GatedMLP(Part):
             self.w_gate_up = ops.interleave_gate_up(g, u)
         else:
             self.w_gate_up = memory.cat([g.to(dt), u.to(dt)], 0, f"{p}gate and up in one matrix")
-        self.w_down = params[p + "down_proj.weight"]
+        self.w_down = params[p + nm["down"]]
 
     def forward(self, ops, step, h, x):
         T = h.shape[0]

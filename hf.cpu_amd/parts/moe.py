@@ -2,7 +2,7 @@
 import torch
 
 from .. import memory
-from ..registry import register_part
+from ..registry import make_part, register_part
 from ..status import EINVAL, ENOTSUP, fail
 from .base import ParamSpec, Part
 
@@ -25,21 +25,27 @@ class MixtureOfExperts(Part):
     ``g = min(Wgate h', limit)``, ``u = clamp(Wup h', -limit, limit)`` (``limit`` <= 0: unbounded), and ``h' = weight_e h``:
     the weight scales the expert's input, not its output (``weight_on="input"``). The gate matrices are named by
     ``names["gate"]``; gate and up of an expert are held as one matrix: in blocks of 32 gate rows and 32 up rows where the
-    expert's size is a multiple of 32 (the up product then forms the activation in its last lines), else gate rows first."""
+    expert's size is a multiple of 32 (the up product then forms the activation in its last lines), else gate rows first.
+    Gated experts with ``weight_on="output"`` are plain gated units whose results are weighted: ``sum_e weight_e Wdown_e (g
+    sigmoid(alpha g) (u + shift))`` with ``g = Wgate h``, ``u = Wup h`` (alpha 1, shift 0: ``silu(g) u``).
+
+    ``scoring="softmax_chosen"``: the ``top`` experts with the largest logits, weighted by the softmax over the chosen logits
+    alone. ``router_bias``: the router's logits are ``Wrouter h + b`` (the tensor named by ``names["router_bias"]``, fp32).
+    ``shared``: the PartSpec of a feed-forward that every token passes beside its experts; its result is added."""
     graph_safe = True
 
     def __init__(self, hidden_size, expert_size, n_experts, top, n_groups=1, keep_groups=1, activation="relu2",
                  scoring="softmax", renormalize=True, weight_scale=1.0, prefix="", names=None, gated=None,
-                 weight_on="output"):
+                 weight_on="output", router_bias=False, shared=None):
         super().__init__(prefix)
-        if weight_on not in ("output", "input") or (weight_on == "input") != (gated is not None):
-            fail(ENOTSUP, "moe: gated experts weigh their input, experts without a gate their output; other pairings are not implemented")
+        if weight_on not in ("output", "input") or (weight_on == "input" and gated is None):
+            fail(ENOTSUP, "moe: experts without a gate weigh their output; gated experts their input or their output")
         self.gated = None if gated is None else (float(gated["alpha"]), float(gated.get("limit", 0.0)), float(gated.get("shift", 0.0)),
                                                  expert_size % 32 == 0)
         self.weight_on = weight_on
         if activation not in ("gelu_erf", "gelu_tanh", "relu2"):
             fail(ENOTSUP, f"moe: activation '{activation}' is not implemented")
-        if scoring not in ("softmax", "sigmoid"):
+        if scoring not in ("softmax", "sigmoid", "softmax_chosen"):
             fail(ENOTSUP, f"moe: scoring '{scoring}' is not implemented")
         if n_experts % n_groups or not 0 < keep_groups <= n_groups:
             fail(EINVAL, f"moe: {n_experts} experts do not form {n_groups} equal groups of which {keep_groups} are kept")
@@ -51,14 +57,22 @@ class MixtureOfExperts(Part):
         self.renormalize, self.weight_scale = bool(renormalize), float(weight_scale)
         self.names = {"router": "router.weight", "up": "experts.{e}.up_proj.weight", "down": "experts.{e}.down_proj.weight",
                       "gate": "experts.{e}.gate_proj.weight"}
+        self.names["router_bias"] = "router.bias"
         self.names.update(names or {})
-        self.w_router = self.w_up = self.w_down = None
+        self.router_bias = bool(router_bias)
+        self.shared = None if shared is None else make_part("feed_forward", shared)
+        self.w_router = self.b_router = self.w_up = self.w_down = None
+
+    def sub_parts(self):
+        return [] if self.shared is None else [self.shared]
 
     def _name(self, key, e=None):
         return self.prefix + (self.names[key] if e is None else self.names[key].format(e=e))
 
     def param_specs(self):
         specs = [ParamSpec(self._name("router"), (self.n_experts, self.E))]
+        if self.router_bias:
+            specs.append(ParamSpec(self._name("router_bias"), (self.n_experts,), "vector", ("normal", 0.1)))
         for e in range(self.n_experts):
             specs += [ParamSpec(self._name("up", e), (self.F, self.E)), ParamSpec(self._name("down", e), (self.E, self.F))]
             if self.gated is not None:
@@ -67,6 +81,7 @@ class MixtureOfExperts(Part):
 
     def bind(self, params, ops):
         self.w_router = params[self._name("router")]
+        self.b_router = params[self._name("router_bias")].contiguous() if self.router_bias else None
         ups = [params.pop(self._name("up", e)) for e in range(self.n_experts)]
         if self.gated is not None:                  # gate and up of an expert in one matrix: one product gives both
             gates = [params.pop(self._name("gate", e)) for e in range(self.n_experts)]
@@ -85,8 +100,11 @@ class MixtureOfExperts(Part):
         T = h.shape[0]
         logits = ops.scratch("router_logits", (T, self.n_experts), torch.float32)
         with ops.section("router"):
-            ops.gemm(h, self.w_router, logits)
+            ops.gemm(h, self.w_router, logits, bias=self.b_router)
             ids, weights = ops.moe_route(logits, self.top, self.n_groups, self.keep_groups, self.scoring, self.renormalize,
                                          self.weight_scale)
         with ops.section("experts"):
-            ops.moe_experts(h, ids, weights, self.w_up, self.w_down, self.activation, x, gated=self.gated)
+            ops.moe_experts(h, ids, weights, self.w_up, self.w_down, self.activation, x, gated=self.gated, weight_on=self.weight_on)
+        if self.shared is not None:
+            with ops.section("shared_expert"):
+                self.shared.forward(ops, step, h, x)

@@ -1,5 +1,6 @@
 """Norms of the residual stream: root mean square with a learned scale (whole, or in groups), and layer norm with scale
 and shift."""
+from .. import memory
 from ..registry import register_part
 from ..status import EINVAL, fail
 from .base import ParamSpec, Part
@@ -13,19 +14,24 @@ class RMSNorm(Part):
     can_be_lazy = True          # forward(..., lazy=True) may leave the division to the products that read the output
 
 
-    def __init__(self, size, eps, prefix="", weight="weight"):
-        """The scale is the tensor ``prefix + weight``."""
+    def __init__(self, size, eps, prefix="", weight="weight", scalar=False):
+        """The scale is the tensor ``prefix + weight``; ``scalar``: a single number for all coordinates (a tensor without
+        dimensions), held as a vector of that number."""
         super().__init__(prefix)
         self.size = size
         self.eps = float(eps)
         self.name = prefix + weight
+        self.scalar = bool(scalar)
         self.weight = None
 
     def param_specs(self):
-        return [ParamSpec(self.name, (self.size,), "vector", ("one_plus_normal", 0.1))]
+        return [ParamSpec(self.name, () if self.scalar else (self.size,), "vector", ("one_plus_normal", 0.1))]
 
     def bind(self, params, ops):
         self.weight = params[self.name]
+        if self.scalar:
+            self.weight = memory.to_device(self.weight.reshape(1).expand(self.size).contiguous(), ops.device,
+                                           f"{self.name}, once a coordinate")
 
     def forward(self, ops, x, out, rows=None, lazy=False):
         """``out[r] = norm(x[rows[r]])`` (``rows`` None: every row in order). ``lazy``: the caller promises that

@@ -1,5 +1,7 @@
 """Position encodings. They act on the packed query/key/value rows of a step and
 hand keys and values to the cache in the same pass."""
+import math
+
 import torch
 
 from .. import memory
@@ -16,12 +18,22 @@ class Rotary(Part):
     reference builds the angle by a running fp32 product, here it is one fp32
     product of the position and a table rounded from fp64). Dimensions from
     ``rot_dim`` on pass through. Values are not rotated; keys are stored rotated
-    (src/model.c:596-600). ``pairing`` ``interleaved``: the pairs are ``(2i, 2i + 1)``, the angles the same."""
+    (src/model.c:596-600). ``pairing`` ``interleaved``: the pairs are ``(2i, 2i + 1)``, the angles the same.
+
+    ``scaling`` = dict(factor, low, high, original) rescales the frequencies by their wavelength ``l = 2 pi / f`` against a
+    context of ``original`` positions: ``f`` stays where ``l < original / high``, becomes ``f / factor`` where ``l > original / low``,
+    and in between is ``(1 - s) f / factor + s f`` with ``s = (original / l - low) / (high - low)`` (computed in fp64, as the
+    frequencies are, then rounded)."""
     graph_safe = True
 
 
-    def __init__(self, head_dim, rot_dim, theta, pairing="split_half", prefix=""):
+    def __init__(self, head_dim, rot_dim, theta, pairing="split_half", prefix="", scaling=None):
         super().__init__(prefix)
+        self.scaling = None
+        if scaling is not None:
+            self.scaling = tuple(float(scaling[k]) for k in ("factor", "low", "high", "original"))
+            if not (self.scaling[0] > 0.0 and self.scaling[2] > self.scaling[1] and self.scaling[3] > 0.0 and self.scaling[1] > 0.0):
+                fail(EINVAL, f"rotary scaling {scaling!r}: factor, low and original must be positive and high above low")
         if pairing not in ("split_half", "interleaved"):
             fail(EINVAL, f"rotary pairing '{pairing}' is not implemented")
         self.pairing = pairing
@@ -36,9 +48,15 @@ class Rotary(Part):
         def table():
             i = torch.arange(self.rot_dim // 2, dtype=torch.float64)
             inv = torch.pow(torch.tensor(self.theta, dtype=torch.float64), -2.0 * i / self.rot_dim)
+            if self.scaling is not None:
+                factor, low, high, original = self.scaling
+                wavelength = 2.0 * math.pi / inv
+                s = (original / wavelength - low) / (high - low)
+                blend = (1.0 - s) * inv / factor + s * inv
+                inv = torch.where(wavelength < original / high, inv, torch.where(wavelength > original / low, inv / factor, blend))
             return memory.to_device(inv.to(torch.float32), ops.device, "rotary frequencies")
         # layers with the same rotation share one table (and with it what a step derives from it once for all of them)
-        self.inv_freq = ops.shared(("rotary frequencies", self.rot_dim, self.theta), table)
+        self.inv_freq = ops.shared(("rotary frequencies", self.rot_dim, self.theta, self.scaling), table)
 
     def store(self, ops, step, qkv, n_heads, n_kv_heads, cache, write, v_head_dim=None, prepare=None):
         """Rotates the queries (and keys) inside ``qkv`` at each token's position;

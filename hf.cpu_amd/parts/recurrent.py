@@ -1,5 +1,6 @@
 """Mixers that keep per-request state of fixed size instead of a growing cache: a state-space layer, linear
-attention with a fixed decay, a matrix memory with exponential gates, and the gated delta rule. All walk a request's
+attention with a fixed decay, a matrix memory with exponential gates, recurrences with a decay per key channel (a forget gate
+that also writes; gated linear attention), and the gated delta rule. All walk a request's
 tokens in order from the state the step before left. The first three share one kernel for the recurrence
 (``Ops.linear_scan``): ``S <- a_t S + k_t (b_t v_t)^T``, ``y_t = S^T q_t + d v_t``; the delta rule, whose write depends on
 what the state already holds along the key, has its own (``Ops.delta_scan``). ``side_by_side`` runs two mixers on one
@@ -323,18 +324,149 @@ class GatedDelta(Part):
                 ops.gemm(normed, self.w_o, x)
 
 
+@register_part("mixer", "hgrn2")
+class ForgetGateRecurrence(Part):
+    """Linear attention in which the forget gate also decides what is written: ``q = silu(Wq h)`` (``n_heads`` x ``head_dim``),
+    ``v = Wv h`` (``n_heads`` x ``v_head_dim``), a forget gate per head and channel ``f = l + (1 - l) sigmoid(Wf h + b)`` with the
+    lower bound ``l`` (tensor ``lower``, one value a (head, channel)); per head ``S_t = diag(f_t) S_(t-1) + (1 - f_t) v_t^T``,
+    ``o_t = S_t^T q_t`` (no key, no other scale). Each head's ``o`` is RMS-normed over ``v_head_dim`` with a weight of that size
+    which all heads share, and the heads are projected. The gate, its complement, the state and the recurrence are fp32; the
+    state lives in the request's state row. ``names``: the tensors' names after ``prefix`` (keys q, v, f, f_bias, lower, norm, o).
+    ``forward(..., accumulate=False)`` writes ``x = ...`` instead of adding."""
+    graph_safe = True
+    can_overwrite = True
+
+    def __init__(self, hidden_size, n_heads, head_dim, v_head_dim, eps, prefix="", names=None):
+        super().__init__(prefix)
+        self.E, self.H, self.D, self.Dv, self.eps = hidden_size, n_heads, head_dim, v_head_dim, float(eps)
+        self.names = dict(q="q", v="v", f="f", f_bias="f.b", lower="lower", norm="norm", o="o")
+        self.names.update(names or {})
+        self.w_in = self.w_o = self.f_bias = self.lower = self.norm_w = None
+
+    def param_specs(self):
+        p, nm = self.prefix, self.names
+        QD, VD = self.H * self.D, self.H * self.Dv
+        return [ParamSpec(p + nm["q"], (QD, self.E)), ParamSpec(p + nm["f"], (QD, self.E)), ParamSpec(p + nm["v"], (VD, self.E)),
+                ParamSpec(p + nm["f_bias"], (QD,), "vector", ("normal", 0.5)), ParamSpec(p + nm["lower"], (QD,), "vector", ("normal", 0.2)),
+                ParamSpec(p + nm["norm"], (self.Dv,), "vector", ("one_plus_normal", 0.1)), ParamSpec(p + nm["o"], (self.E, VD))]
+
+    def cache_need(self):
+        return FixedState(Ops.scan_state_floats(self.H, self.D, self.Dv))
+
+    def bind(self, params, ops):
+        p, nm = self.prefix, self.names
+        mats = [params[p + nm[n]] for n in ("q", "f", "v")]
+        dt = torch.float32 if any(m.dtype == torch.float32 for m in mats) else mats[0].dtype
+        self.w_in = memory.cat([m.to(dt) for m in mats], 0, f"{p}q, the forget gate and v in one matrix")
+        self.w_o = params[p + nm["o"]]
+        self.f_bias, self.lower = params[p + nm["f_bias"]].contiguous(), params[p + nm["lower"]].contiguous()
+        self.norm_w = memory.cat([params[p + nm["norm"]]] * self.H, 0, f"{p}the heads' norm weight, once a head")
+
+    def forward(self, ops, step, h, cache, x, write_cache=True, accumulate=True):
+        if not write_cache:
+            fail(EINVAL, f"hgrn2 '{self.prefix}': a state cannot be read without being advanced")
+        T, QD, VD = h.shape[0], self.H * self.D, self.H * self.Dv
+        proj = ops.scratch("forget_in", (T, 2 * QD + VD), ops.act_dtype)
+        with ops.section("forget_in"):
+            ops.gemm(h, self.w_in, proj)
+        o = ops.scratch("forget_o", (T, VD), torch.float32)
+        with ops.section("forget_scan"):
+            ops.channel_scan(proj[:, :QD], None, proj[:, 2 * QD:], self.H, self.D, self.Dv, proj[:, QD:2 * QD], self.f_bias, cache.state,
+                             step, o, lower=self.lower, q_act="silu")
+        normed = ops.scratch("forget_normed", (T, VD), ops.act_dtype)
+        with ops.section("forget_norm"):
+            ops.group_rmsnorm(o, self.norm_w, self.eps, self.H, normed)
+        with ops.section("forget_wo"):
+            if accumulate:
+                ops.gemm(normed, self.w_o, x, accumulate=True, defer=True)
+            else:
+                ops.gemm(normed, self.w_o, x)
+
+
+@register_part("mixer", "gla")
+class GatedLinearAttention(Part):
+    """Linear attention with a decay per key channel: ``q = Wq h / sqrt(head_dim)``, ``k = Wk h`` (``n_heads`` x ``head_dim``),
+    ``v = Wv h`` (``n_heads`` x ``v_head_dim``), ``alpha = sigmoid(z)^(1 / tau)`` with ``z = Wa2 (Wa1 h) + b`` (a low-rank projection,
+    one value a (head, key channel)); per head ``S_t = diag(alpha_t) S_(t-1) + k_t v_t^T``, ``o_t = S_t^T q_t``. Each head's ``o``
+    is RMS-normed over ``v_head_dim`` with a weight of that size which all heads share; the heads are multiplied by
+    ``silu(Wg h)`` and projected. The decay (from ``z``'s 32-bit sums on: bias, logarithm of the sigmoid, the power), the state and
+    the recurrence are fp32. ``names``: the tensors' names after ``prefix`` (keys q, k, v, g, o, norm, a1, a2, a2_bias).
+    ``forward(..., accumulate=False)`` writes ``x = ...`` instead of adding."""
+    graph_safe = True
+    can_overwrite = True
+
+    def __init__(self, hidden_size, n_heads, head_dim, v_head_dim, tau, eps, decay_rank=None, prefix="", names=None):
+        """``decay_rank``: the inner size of the decay's low-rank projection (None: taken from the tensors)."""
+        super().__init__(prefix)
+        if not tau > 0.0:
+            fail(EINVAL, f"gla: tau {tau} must be positive")
+        self.E, self.H, self.D, self.Dv = hidden_size, n_heads, head_dim, v_head_dim
+        self.tau, self.eps, self.ra = float(tau), float(eps), decay_rank or None
+        self.names = dict(q="q", k="k", v="v", g="g", o="o", norm="norm", a1="a1", a2="a2", a2_bias="a2.b")
+        self.names.update(names or {})
+        self.w_in = self.w_a2 = self.w_o = self.a_bias = self.norm_w = None
+
+    def param_specs(self):
+        p, nm = self.prefix, self.names
+        QD, VD, ra = self.H * self.D, self.H * self.Dv, self.ra or 0
+        return [ParamSpec(p + nm["q"], (QD, self.E)), ParamSpec(p + nm["k"], (QD, self.E)), ParamSpec(p + nm["v"], (VD, self.E)),
+                ParamSpec(p + nm["g"], (VD, self.E)), ParamSpec(p + nm["a1"], (ra, self.E)),
+                ParamSpec(p + nm["a2"], (QD, ra), "matrix", ("normal", 0.1)), ParamSpec(p + nm["a2_bias"], (QD,), "vector", ("normal", 0.5)),
+                ParamSpec(p + nm["norm"], (self.Dv,), "vector", ("one_plus_normal", 0.1)), ParamSpec(p + nm["o"], (self.E, VD))]
+
+    def cache_need(self):
+        return FixedState(Ops.scan_state_floats(self.H, self.D, self.Dv))
+
+    def bind(self, params, ops):
+        p, nm = self.prefix, self.names
+        mats = [params[p + nm[n]] for n in ("q", "k", "v", "g", "a1")]
+        dt = torch.float32 if any(m.dtype == torch.float32 for m in mats) else mats[0].dtype
+        self.w_in = memory.cat([m.to(dt) for m in mats], 0, f"{p}q, k, v, the gate and the decay's first half in one matrix")
+        self.ra = mats[4].shape[0]
+        self.w_a2, self.w_o = params[p + nm["a2"]], params[p + nm["o"]]
+        if self.w_a2.shape[1] != self.ra:
+            fail(EINVAL, f"gla '{p}': the decay's low-rank projection has inner sizes {self.ra} and {self.w_a2.shape[1]}")
+        self.a_bias = params[p + nm["a2_bias"]].contiguous()
+        self.norm_w = memory.cat([params[p + nm["norm"]]] * self.H, 0, f"{p}the heads' norm weight, once a head")
+
+    def forward(self, ops, step, h, cache, x, write_cache=True, accumulate=True):
+        if not write_cache:
+            fail(EINVAL, f"gla '{self.prefix}': a state cannot be read without being advanced")
+        T, QD, VD = h.shape[0], self.H * self.D, self.H * self.Dv
+        proj = ops.scratch("gla_in", (T, 2 * QD + 2 * VD + self.ra), ops.act_dtype)
+        z = ops.scratch("gla_decay", (T, QD), torch.float32)
+        with ops.section("gla_in"):
+            ops.gemm(h, self.w_in, proj)
+            ops.gemm(proj[:, 2 * QD + 2 * VD:], self.w_a2, z)
+        o = ops.scratch("gla_o", (T, VD), torch.float32)
+        with ops.section("gla_scan"):
+            ops.channel_scan(proj[:, :QD], proj[:, QD:2 * QD], proj[:, 2 * QD:2 * QD + VD], self.H, self.D, self.Dv, z, self.a_bias,
+                             cache.state, step, o, tau=self.tau, q_scale=self.D ** -0.5)
+        normed = ops.scratch("gla_normed", (T, VD), ops.act_dtype)
+        with ops.section("gla_norm"):
+            ops.group_rmsnorm(o, self.norm_w, self.eps, self.H, normed, gate=proj[:, 2 * QD + VD:2 * QD + 2 * VD], gate_kind="silu_after")
+        with ops.section("gla_wo"):
+            if accumulate:
+                ops.gemm(normed, self.w_o, x, accumulate=True, defer=True)
+            else:
+                ops.gemm(normed, self.w_o, x)
+
+
 @register_part("mixer", "side_by_side")
 class SideBySide(Part):
     """Two mixers that read the same input; the result is ``scale * (norm_l(left(h)) + norm_r(right(h)))``, each side RMS-normed
     over the model's width with a weight of its own (``names``: keys left_norm, right_norm, after ``prefix``) before the sum
     (``scale`` 0.5: half the sum). ``left`` and ``right`` are PartSpecs of mixers; their caches are this mixer's, by the names
-    ``left`` and ``right``. The sides' results, the norms and the sum are fp32."""
+    ``left`` and ``right``. The sides' results, the norms and the sum are fp32. ``normed=False``: no norms and no weights; the result
+    is the weighted sum ``left_scale * left(h) + right_scale * right(h)``."""
     graph_safe = True
     can_overwrite = True
 
-    def __init__(self, hidden_size, left, right, eps, scale=0.5, prefix="", names=None):
+    def __init__(self, hidden_size, left, right, eps=1e-6, scale=0.5, prefix="", names=None, normed=True, left_scale=1.0, right_scale=1.0):
         super().__init__(prefix)
         self.E, self.eps, self.scale = hidden_size, float(eps), float(scale)
+        self.normed = bool(normed)
+        self.side_scale = {"left": float(left_scale), "right": float(right_scale)}
         self.left, self.right = make_part("mixer", left), make_part("mixer", right)
         self.names = {"left_norm": "left.out", "right_norm": "right.out"}
         self.names.update(names or {})
@@ -345,13 +477,16 @@ class SideBySide(Part):
         return [self.left, self.right]
 
     def param_specs(self):
+        if not self.normed:
+            return []
         return [ParamSpec(self.prefix + self.names[n], (self.E,), "vector", ("one_plus_normal", 0.1)) for n in ("left_norm", "right_norm")]
 
     def cache_need(self):
         return {"left": self.left.cache_need(), "right": self.right.cache_need()}
 
     def bind(self, params, ops):
-        self.w_left, self.w_right = params[self.prefix + self.names["left_norm"]], params[self.prefix + self.names["right_norm"]]
+        if self.normed:
+            self.w_left, self.w_right = params[self.prefix + self.names["left_norm"]], params[self.prefix + self.names["right_norm"]]
         self.short_request_rows = max(getattr(self.left, "short_request_rows", 0), getattr(self.right, "short_request_rows", 0))
 
     def forward(self, ops, step, h, cache, x, write_cache=True, accumulate=True):
@@ -365,4 +500,7 @@ class SideBySide(Part):
                 y.zero_()
                 side.forward(ops, step, h, cache[name], y, write_cache)
             with ops.section("side_norm"):
-                ops.rmsnorm_add(y, w, self.eps, x, scale=self.scale, accumulate=accumulate or name == "right")
+                if self.normed:
+                    ops.rmsnorm_add(y, w, self.eps, x, scale=self.scale, accumulate=accumulate or name == "right")
+                else:
+                    ops.scale_add(y, x, scale=self.side_scale[name], accumulate=accumulate or name == "right")
