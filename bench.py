@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L] [--no-points]
     python bench.py --workload 0.5b | 32b      (the baseline's other workloads, through the scheduler)
-    python bench.py --design goridra | tobozen | mobupel [--sizes 2k,4k] [--batches 8,64] [--context 2048]
+    python bench.py --design goridra | tobozen | mobupel | gitasun [--sizes 2k,4k] [--batches 8,64] [--context 2048]
                                                (another design beside the closest one at equal sizes, part by part; see hf.cpu_amd/bench_design.py)
 
 A step is one decode step of ``--batch`` sequences (default 8) whose prompts of 2,048
@@ -192,7 +192,7 @@ def main():
                     help="for --workload 0.5b | 32b: sample at this temperature (top-k 40, top-p 0.95, min-p 0.05) instead of greedy")
     ap.add_argument("--budget", type=int, default=0,
                     help="for --workload 0.5b | 32b: the scheduler's token budget of a step (0 = the workload's own)")
-    ap.add_argument("--design", choices=["goridra", "tobozen", "mobupel"], default=None,
+    ap.add_argument("--design", choices=["goridra", "tobozen", "mobupel", "gitasun"], default=None,
                     help="measure this design at a few sizes beside Qwen2 dense at equal sizes, every part against its roofline "
                          "(one JSON line a size; --sizes, --batches, --context, --steps apply)")
     ap.add_argument("--sizes", default="", help="with --design: which of its sizes, comma separated (default: all)")

@@ -1,6 +1,6 @@
-"""``bench.py --design goridra | tobozen | mobupel``: prefill and decode of a design at sizes that resemble a real model's layers
+"""``bench.py --design goridra | tobozen | mobupel | gitasun``: prefill and decode of a design at sizes that resemble a real model's layers
 (random weights), beside the closest other design at equal width, heads and layer count (Goridra beside Qwen2 dense,
-Tobozen beside Goridra, Mobupel beside Tobozen), with every part of a step priced against its roofline: flops / time against the matrix cores
+Tobozen beside Goridra, Mobupel and Gitasun beside Tobozen), with every part of a step priced against its roofline: flops / time against the matrix cores
 for a prefill's parts, bytes / time against HBM for a decode step's. One JSON line a size."""
 import json
 import math
@@ -12,12 +12,15 @@ MFMA_PEAK = 2.5e15
 PROMPT, PAGE = 2048, 16
 
 # width, heads, key/value heads, head size, dense ff, experts, choices, groups, kept groups, expert ff, layers, vocabulary
-# (for Tobozen also: heads, head size, state and groups of the state-space layers; layers come in threes)
+# (for Tobozen also: heads, head size, state and groups of the state-space layers; layers come in threes; for Gitasun also the rotated
+# part, the key/value latent and the query latent of its attention through latents)
 SIZES = {
     "2k": dict(width=2048, heads=16, kv_heads=4, dim=128, ff=8192, experts=32, top=4, groups=4, keep=2, expert_ff=1024,
-               layers=8, vocab=32000, mask=1024, ssm_heads=64, ssm_dim=64, ssm_state=128, ssm_groups=8, triples=2),
+               layers=8, vocab=32000, mask=1024, ssm_heads=64, ssm_dim=64, ssm_state=128, ssm_groups=8, triples=2,
+               latent_rot=64, latent_rank=512, latent_q=1536),
     "4k": dict(width=4096, heads=32, kv_heads=8, dim=128, ff=14336, experts=64, top=8, groups=8, keep=4, expert_ff=1024,
-               layers=4, vocab=32000, mask=1024, ssm_heads=128, ssm_dim=64, ssm_state=128, ssm_groups=8, triples=1),
+               layers=4, vocab=32000, mask=1024, ssm_heads=128, ssm_dim=64, ssm_state=128, ssm_groups=8, triples=1,
+               latent_rot=64, latent_rank=512, latent_q=1536),
 }
 
 
@@ -99,6 +102,53 @@ def mobupel_work(z, T, batch, ctx):
     return pre, dec
 
 
+def gitasun_shape(z):
+    """Layers in threes: attention through latents, a forget-gate recurrence, and two mixers side by side (attention with
+    sigmoid weights; gated linear attention); each with a mixture of gated experts and a shared expert."""
+    H, G, D, W = z["heads"], z["kv_heads"], z["dim"], z["width"]
+    moe = dict(kind="moe", expert=dict(ff=z["expert_ff"]), router=dict(experts=z["experts"], top=z["top"]), shared=dict(ff=z["expert_ff"]))
+    R, C = z["latent_rot"], z["latent_rank"]
+    three = [
+        dict(type="latent_attention", mixer=dict(heads=H, dim=D, rot_dim=R, vdim=D, kv_rank=C, q_rank=z["latent_q"], scale=1.0 / math.sqrt(D + R),
+                                                 rot=dict(dims=R, base=10000.0)), mlp=moe),
+        dict(type="hgrn2", mixer=dict(heads=H, dim=D, vdim=D), mlp=moe),
+        dict(type="parallel", mixer=dict(
+            left=dict(heads=H, kv_heads=G, dim=D, vdim=D, scale=1.0 / math.sqrt(D), softcap=30.0,
+                      rot=dict(dims=D, base=500000.0, scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192))),
+            right=dict(heads=H, dim=D, vdim=D, tau=16.0, decay_rank=16), left_scale=0.6, right_scale=1.1), mlp=moe)]
+    return dict(architecture="Gitasun", vocab=z["vocab"], width=W, embedding=dict(scale=math.sqrt(W)), residual_mult=0.7, norm=dict(eps=1e-6),
+                layers=three * z["triples"])
+
+
+def gitasun_work(z, T, batch, ctx):
+    """({part: flops of a prefill of T tokens}, {part: bytes of a decode step}), all layers together, bf16. Attention through
+    latents is priced as the engine computes it, H query heads on one key/value head of R + C key and C value dimensions; the
+    recurrences by the products of their state updates and outputs (4 N P a head and token) in a prefill and by their fp32
+    states, read and written once a request, in a decode step."""
+    W, H, G, D, V, n3 = z["width"], z["heads"], z["kv_heads"], z["dim"], z["vocab"], z["triples"]
+    R, C, Q = z["latent_rot"], z["latent_rank"], z["latent_q"]
+    QD, KD = H * D, G * D
+    E, top, F = z["experts"], z["top"], z["expert_ff"]
+    L = 3 * n3
+    params = {"latent_down": n3 * W * (Q + C + R + QD), "latent_q": n3 * Q * H * (D + R), "latent_pack": n3 * H * D * C, "latent_v": n3 * H * D * C,
+              "latent_wo": n3 * QD * W, "qkv": n3 * W * (2 * QD + 2 * KD), "wo": n3 * QD * W, "forget_in": n3 * W * 3 * QD, "forget_wo": n3 * QD * W,
+              "gla_in": n3 * (W * (4 * QD + 16) + 16 * QD), "gla_wo": n3 * QD * W, "router": L * E * W, "shared_expert": L * 3 * F * W, "head": V * W}
+    pre = {k: 2.0 * T * v for k, v in params.items() if k != "head"}
+    pre["latent_attn"] = n3 * 2.0 * (R + 2 * C) * H * T * (T + 1) / 2
+    pre["attn"] = n3 * 4.0 * D * H * T * (T + 1) / 2
+    pre["forget_scan"] = n3 * T * H * 4.0 * D * D
+    pre["gla_scan"] = n3 * T * H * 4.0 * D * D
+    pre["experts"] = L * T * top * 6.0 * F * W
+    dec = {k: 2.0 * v for k, v in params.items()}
+    touched = E * (1.0 - (1.0 - top / E) ** batch)
+    dec["experts"] = L * touched * 3 * F * W * 2.0
+    dec["latent_attn"] = batch * ctx * n3 * 2.0 * (R + 2 * C)
+    dec["attn"] = batch * ctx * n3 * 2.0 * 2 * KD
+    dec["forget_scan"] = batch * n3 * H * D * D * 4 * 2.0
+    dec["gla_scan"] = batch * n3 * H * D * D * 4 * 2.0
+    return pre, dec
+
+
 def goridra_shape(z):
     """Layers in pairs: one with keys and values of its own and a dense feed-forward, one that reads them and has
     a mixture of experts."""
@@ -135,6 +185,8 @@ def part_work(design, z, T, batch, ctx):
         return tobozen_work(z, T, batch, ctx)
     if design == "mobupel":
         return mobupel_work(z, T, batch, ctx)
+    if design == "gitasun":
+        return gitasun_work(z, T, batch, ctx)
     W, H, G, D, L, V = z["width"], z["heads"], z["kv_heads"], z["dim"], z["layers"], z["vocab"]
     QD, KD = H * D, G * D
     if design == "qwen2":
@@ -171,9 +223,9 @@ def run(args):
     for size in (args.sizes.split(",") if args.sizes else list(SIZES)):
         z = SIZES[size]
         line = {"size": size, "dims": z, "context": context, "dtype": "bf16", "data": "synthetic"}
-        shapes = {"goridra": goridra_shape, "qwen2": qwen2_shape, "tobozen": tobozen_shape, "mobupel": mobupel_shape}
-        beside = {"goridra": "qwen2", "tobozen": "goridra", "mobupel": "tobozen"}[args.design]
-        if args.design in ("tobozen", "mobupel"):    # the same number of layers in both designs
+        shapes = {"goridra": goridra_shape, "qwen2": qwen2_shape, "tobozen": tobozen_shape, "mobupel": mobupel_shape, "gitasun": gitasun_shape}
+        beside = {"goridra": "qwen2", "tobozen": "goridra", "mobupel": "tobozen", "gitasun": "tobozen"}[args.design]
+        if args.design in ("tobozen", "mobupel", "gitasun"):    # the same number of layers in both designs
             z = dict(z, layers=3 * z["triples"])
         for design, shape in ((args.design, shapes[args.design](z)), (beside, shapes[beside](z))):
             cfg = hf_cpu_amd.config_from_dict(shape)

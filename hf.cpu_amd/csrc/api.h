@@ -101,7 +101,7 @@ int hfa_attention_prompt_rows(void);
 // of head h being its weights on the values of group (h's group + r) mod G (see hfa_talk_mix; on the matrix cores one pass a round).
 // `softcap` > 0: score <- softcap tanh(score / softcap) before the weights are formed. `weights` 0: softmax; 1: no softmax, a
 // visible key weighs sigmoid(score + head_bias[h]) (head_bias: one fp32 per query head, or null), not normalised over the keys.
-// Both go the plain way.
+// Sigmoid weights (with or without a cap) run on the matrix cores under the same conditions as the softmax; a cap under a softmax goes the plain way.
 int hfa_paged_attention(const void* q, int dtype, int ldq, const void* k_cache, const void* v_cache,
                         int kv_width, int v_width, const int* block_table, int max_blocks, const int* token_slot,
                         const int* positions, const int* q_start, int n_seqs, int max_q_len, int max_seq_len,

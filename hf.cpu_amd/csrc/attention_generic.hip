@@ -234,12 +234,13 @@ extern "C" int hfa_paged_attention(const void* q, int dtype, int ldq, const void
     HFA_REQUIRE(dtype == HFA_F32 || dtype == HFA_BF16, "paged_attention: unknown dtype %d", dtype);
     AttnArgs a = {q, ldq, k_cache, v_cache, kv_width, block_table, max_blocks, token_slot, positions, q_start,
                   n_seqs, max_q_len, max_seq_len, out, ldo, n_tokens, n_heads, n_kv_heads, head_dim, page_tokens,
-                  window, scale, workspace, workspace_bytes, stream, nullptr, 0, nullptr, nullptr, mask_chunk, sink ? 1 : 0, 0};
+                  window, scale, workspace, workspace_bytes, stream, nullptr, 0, nullptr, nullptr, mask_chunk, sink ? 1 : 0, 0,
+                  softcap, weights, head_bias};
     // the matrix-core kernels take no slopes: scores with a position term go the plain way
     // and they know one head size and one row width for keys and values
     HFA_REQUIRE(softcap >= 0.f && (weights == 0 || weights == 1), "paged_attention: a negative soft cap or an unknown kind of weights");
-    // nor a soft cap on the scores, nor weights that are no softmax
-    if (!force_plain && !slopes && softcap == 0.f && weights == 0 && dtype == HFA_BF16 && v_head_dim == head_dim && v_width == kv_width && attn_mfma_supports(a)) {
+    // nor a soft cap on the scores under a softmax; sigmoid weights (with or without a cap) they take, for a head's own values
+    if (!force_plain && !slopes && (weights == 1 ? !cross_values && !sink : softcap == 0.f) && dtype == HFA_BF16 && v_head_dim == head_dim && v_width == kv_width && attn_mfma_supports(a)) {
         if (!cross_values) return attn_mfma_launch(a);
         // single tokens: one pass over the cache for all rounds
         int chunk_keys = 0, n_chunks = 0;
@@ -256,6 +257,9 @@ extern "C" int hfa_paged_attention(const void* q, int dtype, int ldq, const void
         }
         return 0;
     }
+    // one key/value head with wide keys and values of a size of their own, read by every query head
+    if (!force_plain && !slopes && !cross_values && dtype == HFA_BF16 && attn_shared_supports(a, v_head_dim, v_width))
+        return attn_shared_launch(a, v_head_dim);
     return attn_generic_launch(q, dtype, ldq, k_cache, v_cache, kv_width, v_width, block_table, max_blocks, token_slot,
                                positions, out, ldo, n_tokens, n_heads, n_kv_heads, head_dim, v_head_dim, page_tokens, window,
                                mask_chunk, scale, slopes, sink ? 1 : 0, cross_values ? 1 : 0, softcap, weights, head_bias, stream);

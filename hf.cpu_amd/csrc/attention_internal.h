@@ -21,6 +21,9 @@ struct AttnArgs {
     int mask_chunk;                // > 0: a query sees only the keys of its own run of mask_chunk positions, counted from 0
     int sink;                      // 1: the softmax's denominator holds one more term of score 0 that has no value
     int v_rot;                     // the weights of a head of group c are applied to the values of group (c + v_rot) mod G (0: its own)
+    float softcap;                 // > 0 (with weights 1 only): score <- softcap tanh(score / softcap)
+    int weights;                   // 0: softmax; 1: sigmoid(score + head_bias[head]), not normalised over the keys
+    const float* head_bias;        // one number a query head, or null
 };
 
 // The first key that the query at `pos` sees: a window of the last `window` positions (0: none) and/or the start
@@ -45,6 +48,11 @@ int attn_generic_launch(const void* q, int dtype, int ldq, const void* k_cache, 
 // of the keys that `launch` takes.
 bool attn_cross_supports(const AttnArgs& a, int* chunk_keys, int* n_chunks);
 int attn_cross_launch(const AttnArgs& a, int chunk_keys, int n_chunks);
+
+// Many query heads on one key/value head with wide key rows and value rows of another size (attention through latents), bf16 on
+// the matrix cores; see attention_shared.hip for what it needs.
+bool attn_shared_supports(const AttnArgs& a, int v_head_dim, int v_width);
+int attn_shared_launch(const AttnArgs& a, int v_head_dim);
 
 // bf16 on the matrix cores; see attention_mfma.hip for what it needs.
 bool attn_mfma_supports(const AttnArgs& a);

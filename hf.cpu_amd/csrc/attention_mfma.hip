@@ -71,14 +71,17 @@ union Frag {
 // new key, stores it and the new value into the cache (rows slot_map[token]) for the steps to come, and uses them
 // from LDS itself, since what the cache row held before is not the token's. What rope_store would have done in a
 // kernel and a pass over memory of its own.
-template <int NDB, bool SPLIT, bool FUSED>
+// SIG: the weights are no softmax but sigmoid(capped score + head_bias[head]) (see hfa_paged_attention); records of key
+// chunks then carry maximum 0 and sum 1 in the first chunk and 0 in the others, so that the merge adds the chunks up.
+template <int NDB, bool SPLIT, bool FUSED, bool SIG = false>
 __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
     const uint16_t* __restrict__ q, int ldq, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc, int kvw,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_slot,
     const int* __restrict__ positions, const int* __restrict__ q_start, int n_seqs, uint16_t* __restrict__ out,
     int ldo, float* __restrict__ partial, int H, int psh, int window, int mask_chunk, float scale_log2e, int tpt, int cpt,
     int chunk_keys, int n_chunks, int one_tile_each, const float* __restrict__ raw, int ld_raw,
-    const float* __restrict__ cs, const int* __restrict__ slot_map, int G, int sink, int v_rot) {
+    const float* __restrict__ cs, const int* __restrict__ slot_map, int G, int sink, int v_rot, float softcap = 0.f,
+    const float* __restrict__ head_bias = nullptr) {
     constexpr int D = NDB * 32, KS = D / 16;
     const int P = 1 << psh;                                // tokens per page, a power of two
     const int lane = threadIdx.x, col = lane & 31, half = lane >> 5;
@@ -111,6 +114,7 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
     const bool col_ok = col < n_cols;
     const int my_tok = col_ok ? t0 + col / cpt : t0;
     const int my_head = g * cpt + (col_ok ? col % cpt : 0);
+    const float hb = (SIG && head_bias) ? head_bias[my_head] : 0.f;
     const int pos = positions[my_tok];
     const int pos_first = positions[t0], hi = positions[t_end - 1];
     int k_begin = first_visible(pos_first, window, mask_chunk);
@@ -296,47 +300,60 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
         // Most blocks lie wholly inside what every column of the wave may see (unused columns
         // aside, whose results are dropped): no key of them needs the visibility test, and the
         // scale (positive) moves into the exponent's fma.
-        const bool inside = __all(!col_ok || (key0 >= vlo && key0 + KB - 1 <= vhi)) != 0;
-        float mx = NEG_BIG, mn, corr, psum = 0.f;
-        if (inside) {
-#pragma unroll
-            for (int r = 0; r < 16; r++) mx = fmaxf(mx, st[r]);
-            mx = pair_max(mx) * scale_log2e;
-            mn = mx > m + MAX_SLACK ? mx : m;
-            corr = fast_exp2(m - mn);
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                st[r] = fast_exp2(fmaf(st[r], scale_log2e, -mn));
-                psum += st[r];
-            }
-        } else {
+        if constexpr (SIG) {
+            // no softmax: a visible key weighs sigmoid(score + the head's number), the score capped by c tanh(score / c) =
+            // c (1 - 2 / (1 + exp(2 score / c))) first if a cap is given; no maximum, no sum, nothing to rescale
+            const float sc = scale_log2e * 0.6931471805599453f, cap2 = softcap > 0.f ? 2.885390081777927f / softcap : 0.f;
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int kr = key0 + 8 * (r / 4) + 4 * half + (r % 4);
-                const bool vis = kr >= vlo && kr <= vhi;
-                st[r] = vis ? st[r] * scale_log2e : NEG_BIG;
-                mx = fmaxf(mx, st[r]);
+                float sv = st[r] * sc;
+                if (softcap > 0.f) sv = softcap * (1.0f - 2.0f / (1.0f + fast_exp2(sv * cap2)));
+                st[r] = (kr >= vlo && kr <= vhi) ? 1.0f / (1.0f + fast_exp2(-1.4426950408889634f * (sv + hb))) : 0.f;
             }
-            mx = pair_max(mx);
-            mn = mx > m + MAX_SLACK ? mx : m;
-            corr = fast_exp2(m - mn);
+        } else {
+            const bool inside = __all(!col_ok || (key0 >= vlo && key0 + KB - 1 <= vhi)) != 0;
+            float mx = NEG_BIG, mn, corr, psum = 0.f;
+            if (inside) {
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const float p = st[r] > 0.5f * NEG_BIG ? fast_exp2(st[r] - mn) : 0.f;
-                st[r] = p;
-                psum += p;
+                for (int r = 0; r < 16; r++) mx = fmaxf(mx, st[r]);
+                mx = pair_max(mx) * scale_log2e;
+                mn = mx > m + MAX_SLACK ? mx : m;
+                corr = fast_exp2(m - mn);
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    st[r] = fast_exp2(fmaf(st[r], scale_log2e, -mn));
+                    psum += st[r];
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int kr = key0 + 8 * (r / 4) + 4 * half + (r % 4);
+                    const bool vis = kr >= vlo && kr <= vhi;
+                    st[r] = vis ? st[r] * scale_log2e : NEG_BIG;
+                    mx = fmaxf(mx, st[r]);
+                }
+                mx = pair_max(mx);
+                mn = mx > m + MAX_SLACK ? mx : m;
+                corr = fast_exp2(m - mn);
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const float p = st[r] > 0.5f * NEG_BIG ? fast_exp2(st[r] - mn) : 0.f;
+                    st[r] = p;
+                    psum += p;
+                }
             }
-        }
-        psum = pair_sum(psum);
-        l = l * corr + psum;
-        m = mn;
-        // the running maxima settle after a few blocks; the accumulators are rescaled only when
-        // some column's maximum moved (decided by the whole wave together)
-        if (__any(corr != 1.0f)) {
+            psum = pair_sum(psum);
+            l = l * corr + psum;
+            m = mn;
+            // the running maxima settle after a few blocks; the accumulators are rescaled only when
+            // some column's maximum moved (decided by the whole wave together)
+            if (__any(corr != 1.0f)) {
 #pragma unroll
-            for (int db = 0; db < NDB; db++)
+                for (int db = 0; db < NDB; db++)
 #pragma unroll
-                for (int r = 0; r < 16; r++) o[db][r] *= corr;
+                    for (int r = 0; r < 16; r++) o[db][r] *= corr;
+            }
         }
 #pragma unroll
         for (int kk = 0; kk < 2; kk++) {
@@ -442,6 +459,10 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
     }
 
     if (!col_ok) return;
+    if (SIG) {
+        m = 0.f;
+        l = (!SPLIT || chunk == 0) ? 1.f : 0.f;
+    }
     // element r of o[db]: dimension 32 db + 8 (r / 4) + 4 half + r % 4 of this lane's column
     if (SPLIT) {
         float* dst = partial + ((size_t)(my_tok * H + my_head) * n_chunks + chunk) * (D + 2);
@@ -482,13 +503,14 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
 // are numbered from the end of each request backwards, so the longest ones start first.
 #define PVS 36       // LDS row of a value dimension: 32 keys + 4 pad (elements)
 
-template <int NDB, bool SMALL_PAGES>
+template <int NDB, bool SMALL_PAGES, bool SIG = false>
 __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_kernel(
     const uint16_t* __restrict__ q, int ldq, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc, int kvw,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_slot,
     const int* __restrict__ positions, const int* __restrict__ q_start, int n_seqs, uint16_t* __restrict__ out,
     int ldo, int psh, int window, int mask_chunk, float scale_log2e, int tpt, int cpt, int n_tiles, int pair_from,
-    float* __restrict__ partial, int H, int chunk_keys, int n_chunks, int sink, int v_rot) {
+    float* __restrict__ partial, int H, int chunk_keys, int n_chunks, int sink, int v_rot, float softcap = 0.f,
+    const float* __restrict__ head_bias = nullptr) {
     constexpr int D = NDB * 32, KS = D / 16, KROW = D + 8;
     const int P = 1 << psh;                                // tokens per page, a power of two
     __shared__ __attribute__((aligned(16))) uint16_t k_s[2][KB * KROW];
@@ -537,6 +559,7 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
     const bool col_ok = col < n_cols;
     const int my_tok = col_ok ? w0 + col / cpt : t0;
     const int my_head = g * cpt + (col_ok ? col % cpt : 0);
+    const float hb = (SIG && head_bias) ? head_bias[my_head] : 0.f;
     const int pos = positions[my_tok];
     const int pos_first = positions[t0];
     int hi = positions[t_end - 1];
@@ -714,45 +737,58 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
                 __builtin_amdgcn_sched_barrier(0);
                 // Most blocks lie wholly inside what every column of the wave may see (unused columns
                 // aside, whose results are dropped): no key of them needs the visibility test.
-                const bool inside = __all(!col_ok || (key0 >= vlo && key0 + KB - 1 <= vhi)) != 0;
-                float mx = NEG_BIG, mn, corr, psum = 0.f;
-                if (inside) {                                   // the scale (positive) moves into the exponent's fma
-#pragma unroll
-                    for (int r = 0; r < 16; r++) mx = fmaxf(mx, st[r]);
-                    mx = pair_max(mx) * scale_log2e;
-                    mn = mx > m + MAX_SLACK ? mx : m;
-                    corr = fast_exp2(m - mn);
-#pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        st[r] = fast_exp2(fmaf(st[r], scale_log2e, -mn));
-                        psum += st[r];
-                    }
-                } else {
+                if constexpr (SIG) {
+                    // no softmax: a visible key weighs sigmoid(score + the head's number), the score capped by c tanh(score / c) =
+                    // c (1 - 2 / (1 + exp(2 score / c))) first if a cap is given; no maximum, no sum, nothing to rescale
+                    const float sc = scale_log2e * 0.6931471805599453f, cap2 = softcap > 0.f ? 2.885390081777927f / softcap : 0.f;
 #pragma unroll
                     for (int r = 0; r < 16; r++) {
                         const int kr = key0 + 8 * (r / 4) + 4 * half + (r % 4);
-                        const bool vis = kr >= vlo && kr <= vhi;
-                        st[r] = vis ? st[r] * scale_log2e : NEG_BIG;
-                        mx = fmaxf(mx, st[r]);
+                        float sv = st[r] * sc;
+                        if (softcap > 0.f) sv = softcap * (1.0f - 2.0f / (1.0f + fast_exp2(sv * cap2)));
+                        st[r] = (kr >= vlo && kr <= vhi) ? 1.0f / (1.0f + fast_exp2(-1.4426950408889634f * (sv + hb))) : 0.f;
                     }
-                    mx = pair_max(mx);
-                    mn = mx > m + MAX_SLACK ? mx : m;
-                    corr = fast_exp2(m - mn);
+                } else {
+                    const bool inside = __all(!col_ok || (key0 >= vlo && key0 + KB - 1 <= vhi)) != 0;
+                    float mx = NEG_BIG, mn, corr, psum = 0.f;
+                    if (inside) {                                   // the scale (positive) moves into the exponent's fma
 #pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        const float p = st[r] > 0.5f * NEG_BIG ? fast_exp2(st[r] - mn) : 0.f;
-                        st[r] = p;
-                        psum += p;
+                        for (int r = 0; r < 16; r++) mx = fmaxf(mx, st[r]);
+                        mx = pair_max(mx) * scale_log2e;
+                        mn = mx > m + MAX_SLACK ? mx : m;
+                        corr = fast_exp2(m - mn);
+#pragma unroll
+                        for (int r = 0; r < 16; r++) {
+                            st[r] = fast_exp2(fmaf(st[r], scale_log2e, -mn));
+                            psum += st[r];
+                        }
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 16; r++) {
+                            const int kr = key0 + 8 * (r / 4) + 4 * half + (r % 4);
+                            const bool vis = kr >= vlo && kr <= vhi;
+                            st[r] = vis ? st[r] * scale_log2e : NEG_BIG;
+                            mx = fmaxf(mx, st[r]);
+                        }
+                        mx = pair_max(mx);
+                        mn = mx > m + MAX_SLACK ? mx : m;
+                        corr = fast_exp2(m - mn);
+#pragma unroll
+                        for (int r = 0; r < 16; r++) {
+                            const float p = st[r] > 0.5f * NEG_BIG ? fast_exp2(st[r] - mn) : 0.f;
+                            st[r] = p;
+                            psum += p;
+                        }
                     }
-                }
-                psum = pair_sum(psum);
-                l = l * corr + psum;
-                m = mn;
-                if (__any(corr != 1.0f)) {                      // see above: only when a maximum moved
+                    psum = pair_sum(psum);
+                    l = l * corr + psum;
+                    m = mn;
+                    if (__any(corr != 1.0f)) {                      // see above: only when a maximum moved
 #pragma unroll
-                    for (int db = 0; db < NDB; db++)
+                        for (int db = 0; db < NDB; db++)
 #pragma unroll
-                        for (int r = 0; r < 16; r++) o[db][r] *= corr;
+                            for (int r = 0; r < 16; r++) o[db][r] *= corr;
+                    }
                 }
                 Frag pf[2];
 #pragma unroll
@@ -785,6 +821,10 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
         }
     }
     if (!col_ok) return;
+    if (SIG) {
+        m = 0.f;
+        l = (n_chunks == 1 || blockIdx.z == 0) ? 1.f : 0.f;
+    }
     if (n_chunks > 1) {
         float* dst = partial + ((size_t)(my_tok * H + my_head) * n_chunks + blockIdx.z) * (D + 2);
         if (half == 0) {
@@ -900,7 +940,10 @@ static int launch_ndb(const AttnArgs& a, int tiles, int tpt, int cpt, int chunk_
         a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo, PARTIAL, a.n_heads,         \
         page_shift(a.page_tokens), a.window, a.mask_chunk, sl, tpt, cpt, chunk_keys, n_chunks, a.max_q_len <= tpt, a.raw, a.ld_raw,      \
         a.cos_sin, a.slot_map, a.n_kv_heads, a.sink, a.v_rot
-    if (a.raw) {
+    if (a.weights == 1) {
+        if (n_chunks > 1) attn_mfma_kernel<NDB, true, false, true><<<grid, WAVE, 0, a.stream>>>(ATTN_ARGS((float*)a.workspace), a.softcap, a.head_bias);
+        else attn_mfma_kernel<NDB, false, false, true><<<grid, WAVE, 0, a.stream>>>(ATTN_ARGS(nullptr), a.softcap, a.head_bias);
+    } else if (a.raw) {
         if (n_chunks > 1) attn_mfma_kernel<NDB, true, true><<<grid, WAVE, 0, a.stream>>>(ATTN_ARGS((float*)a.workspace));
         else attn_mfma_kernel<NDB, false, true><<<grid, WAVE, 0, a.stream>>>(ATTN_ARGS(nullptr));
     } else {
@@ -954,18 +997,19 @@ static int launch_prefill(const AttnArgs& a, int tpt, int cpt) {
         pair_from = 0;
         grid.z = n_chunks;
     }
-    if (a.page_tokens <= 32)
-        attn_prefill_kernel<NDB, true><<<grid, 4 * WAVE, 0, a.stream>>>(
-            (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width, a.block_table,
-            a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo,
-            page_shift(a.page_tokens), a.window, a.mask_chunk, a.scale * 1.4426950408889634f, tpt, cpt, n_tiles, pair_from,
-            (float*)a.workspace, a.n_heads, chunk_keys, n_chunks, a.sink, a.v_rot);
+#define PREFILL_ARGS                                                                                                       \
+    (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width, a.block_table,            \
+        a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo, page_shift(a.page_tokens),      \
+        a.window, a.mask_chunk, a.scale * 1.4426950408889634f, tpt, cpt, n_tiles, pair_from, (float*)a.workspace, a.n_heads,   \
+        chunk_keys, n_chunks, a.sink, a.v_rot
+    if (a.weights == 1) {
+        if (a.page_tokens <= 32) attn_prefill_kernel<NDB, true, true><<<grid, 4 * WAVE, 0, a.stream>>>(PREFILL_ARGS, a.softcap, a.head_bias);
+        else attn_prefill_kernel<NDB, false, true><<<grid, 4 * WAVE, 0, a.stream>>>(PREFILL_ARGS, a.softcap, a.head_bias);
+    } else if (a.page_tokens <= 32)
+        attn_prefill_kernel<NDB, true><<<grid, 4 * WAVE, 0, a.stream>>>(PREFILL_ARGS);
     else
-        attn_prefill_kernel<NDB, false><<<grid, 4 * WAVE, 0, a.stream>>>(
-            (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width, a.block_table,
-            a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo,
-            page_shift(a.page_tokens), a.window, a.mask_chunk, a.scale * 1.4426950408889634f, tpt, cpt, n_tiles, pair_from,
-            (float*)a.workspace, a.n_heads, chunk_keys, n_chunks, a.sink, a.v_rot);
+        attn_prefill_kernel<NDB, false><<<grid, 4 * WAVE, 0, a.stream>>>(PREFILL_ARGS);
+#undef PREFILL_ARGS
     HFA_LAUNCH_CHECK("attn_prefill");
     if (n_chunks > 1) {
         attn_merge_kernel<<<dim3(a.n_tokens, a.n_heads), WAVE, 0, a.stream>>>((const float*)a.workspace, (uint16_t*)a.out, a.ldo,

@@ -632,7 +632,7 @@ class Ops:
         round r of head h (at ``(r * heads + h) * v_head_dim``) being its weights on the values of group (h's group + r) mod
         groups (see ``talk_mix``). ``softcap`` c > 0: a score becomes ``c tanh(score / c)`` before the weights are formed.
         ``weights`` ``"sigmoid"``: no softmax; a visible key weighs ``sigmoid(score + head_bias[h])`` (``head_bias``: fp32, one per
-        query head, or None), and the weights are not normalised over the keys. Both take the plain kernel."""
+        query head, or None), and the weights are not normalised over the keys (on the matrix cores where a softmax would be; a cap under a softmax takes the plain kernel)."""
         v_head_dim = head_dim if v_head_dim is None else int(v_head_dim)
         mask_chunk = int(mask_chunk)
         if weights not in ("softmax", "sigmoid") or (weights == "sigmoid" and (sink or cross_values)):
@@ -642,6 +642,7 @@ class Ops:
             fail(EINVAL, "paged_attention: head_bias goes with sigmoid weights and is contiguous fp32 on the device, one per query head")
         softcap = float(softcap or 0.0)
         shaped_scores = softcap != 0.0 or weights != "softmax"
+        plain_scores = softcap != 0.0 and weights == "softmax"        # what only the plain kernel computes
         self._scaled.pop(out.data_ptr(), None)               # whatever `out` held, it is no norm's lazy output any more
         lr = self._lazy_rope
         if lr is not None and lr.qkv.data_ptr() == q.data_ptr() and lr.cache is cache and slopes is None and not sink \
@@ -692,7 +693,7 @@ class Ops:
         # take as long as thousands of prompt tokens). The step lays requests with few tokens first, so
         # each part is a step of its own: the first goes to the kernel that cuts the keys into chunks.
         n_short = getattr(step, "n_short_seqs", 0)
-        if not plain and not shaped_scores and v_head_dim == head_dim and q.dtype == torch.bfloat16 \
+        if not plain and not plain_scores and v_head_dim == head_dim and q.dtype == torch.bfloat16 \
                 and step.max_q_len >= self.prompt_rows and 0 < n_short < step.n_seqs:
             ts = step.n_short_tokens
             _ints(step.q_start_long, "q_start_long", step.n_seqs - n_short + 1)

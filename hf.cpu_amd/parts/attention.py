@@ -378,7 +378,7 @@ class LatentAttention(Part):
                 ops.gemm(q[:, hd * (D + R):hd * (D + R) + D], self.w_uk_t[hd], packed[:, hd * HD + R:(hd + 1) * HD])
             self.position.store(ops, step, packed, H, 1, cache, True, v_head_dim=C)
         att = ops.scratch("latent_att", (T, H * C), ops.act_dtype)
-        with ops.section("attn"):
+        with ops.section("latent_attn"):
             ops.paged_attention(packed, H, 1, HD, cache, step, 0, self.scale, att, v_head_dim=C)
         heads = ops.scratch("att", (T, H * Dv), ops.act_dtype)
         with ops.section("latent_v"):
@@ -386,7 +386,7 @@ class LatentAttention(Part):
                 ops.gemm(att[:, hd * C:(hd + 1) * C], self.w_uv[hd * Dv:(hd + 1) * Dv], heads[:, hd * Dv:(hd + 1) * Dv])
             if self.out_gate:
                 ops.gate_mul(heads, gate, heads, "sigmoid")
-        with ops.section("wo"):
+        with ops.section("latent_wo"):
             if accumulate:
                 ops.gemm(heads, self.w_o, x, accumulate=True, defer=True)
             else:

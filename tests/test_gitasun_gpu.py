@@ -188,7 +188,8 @@ def paged_rows(rng, lengths, kw, vw, page, dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,G,D,Dv,page,cap", [(4, 2, 16, 16, 16, 0.0), (3, 1, 32, 20, 8, 5.0), (8, 8, 64, 64, 16, 30.0), (6, 2, 48, 32, 4, 2.0),
-                                               (6, 1, 48, 32, 16, 30.0), (2, 2, 10, 6, 8, 0.0)])
+                                               (6, 1, 48, 32, 16, 30.0), (2, 2, 10, 6, 8, 0.0), (4, 2, 128, 128, 16, 20.0), (6, 1, 32, 32, 8, 0.0),
+                                               (8, 2, 64, 64, 32, 0.0), (16, 4, 96, 96, 16, 50.0)])
 def test_attention_with_capped_scores_and_sigmoid_weights(ops32, dtype, H, G, D, Dv, page, cap):
     """Queries at the last positions of each request (a portion for some, a single token for others): every visible key
     weighs sigmoid(cap tanh(score / cap) + b_h), not normalised; a key far back, one at a page's last place and the
@@ -236,6 +237,100 @@ def test_attention_with_capped_scores_and_sigmoid_weights(ops32, dtype, H, G, D,
         step1 = FakeStep(ints([n - 1]), ints([s]), table, None)
         ops32.paged_attention(dev(qs[s][-1:].reshape(1, H * D), dtype), H, G, D, cache, step1, 0, scale * 3.0, out1, v_head_dim=Dv, softcap=cap)
         assert np.max(np.abs(out1.float().cpu().numpy() - want1)) <= (2e-5 if dtype == torch.float32 else 0.02)
+
+
+@pytest.mark.parametrize("H,G,D,page,cap,lengths,q_lens", [
+    (8, 2, 64, 16, 30.0, [700, 1500], [1, 1]),              # single tokens: the keys cut into chunks, the chunks' sums added
+    (16, 4, 128, 16, 0.0, [3000, 40, 1], [1, 1, 1]),
+    (4, 1, 32, 8, 10.0, [1500], [64]),                      # a portion far into a prompt: few blocks, each cut into chunks
+    (8, 4, 64, 16, 30.0, [900, 333], [900, 333]),           # whole prompts
+    (8, 2, 128, 64, 5.0, [1100, 17], [300, 17]),
+])
+def test_sigmoid_weights_on_the_matrix_cores_at_long_contexts(ops16, H, G, D, page, cap, lengths, q_lens):
+    """The matrix-core kernels' own cuttings (key chunks for few queries, four waves a tile for portions) against the
+    plain kernel on the same cache, and against float64 for the last token of each request."""
+    rng = np.random.default_rng(H + D + sum(lengths))
+    ks, vs, cache, table = paged_rows(rng, lengths, G * D, G * D, page, torch.bfloat16)
+    bias = (rng.standard_normal(H) - 4.0).astype(np.float32)
+    scale = 1.0 / math.sqrt(D)
+    qs, positions, slots = [], [], []
+    for s, (n, ql) in enumerate(zip(lengths, q_lens)):
+        q = rng.standard_normal((ql, H, D)).astype(np.float32)
+        if n > 100:
+            q[-1] += 4.0 * np.repeat(ks[s][2].reshape(G, D), H // G, axis=0) / math.sqrt(D)      # a key far back stands out
+        qs.append(q)
+        positions += list(range(n - ql, n))
+        slots += [s] * ql
+    q = dev(np.concatenate(qs).reshape(-1, H * D), torch.bfloat16)
+    step = FakeStep(ints(positions), ints(slots), table, None)
+    out, other = torch.empty_like(q), torch.empty_like(q)
+    args = dict(softcap=cap, weights="sigmoid", head_bias=dev(bias))
+    ops16.paged_attention(q, H, G, D, cache, step, 0, scale, out, **args)
+    ops16.force_plain_attention = True
+    try:
+        ops16.paged_attention(q, H, G, D, cache, step, 0, scale, other, **args)
+    finally:
+        ops16.force_plain_attention = False
+    got, plain_got = out.float().cpu().numpy(), other.float().cpu().numpy()
+    assert np.max(np.abs(got - plain_got) / (np.abs(plain_got) + 1.0)) <= 0.03            # (probabilities rounded to bf16 on the matrix cores)
+    grp = np.arange(H) // (H // G)
+    at = 0
+    for s, (n, ql) in enumerate(zip(lengths, q_lens)):
+        at += ql
+        k, v = rounded(ks[s], torch.bfloat16).reshape(n, G, D), rounded(vs[s], torch.bfloat16).reshape(n, G, D)
+        sc = np.einsum("hd,jhd->hj", rounded(qs[s][-1], torch.bfloat16), k[:, grp]) * scale
+        if cap:
+            sc = cap * np.tanh(sc / cap)
+        want = np.einsum("hj,jhd->hd", pg.sigmoid(sc + bias[:, None].astype(np.float64)), v[:, grp]).reshape(-1)
+        assert np.max(np.abs(got[at - 1] - want) / (np.abs(want) + 1.0)) <= 0.02, f"request {s}"
+
+
+@pytest.mark.parametrize("H,DK,C,page,lengths,q_lens", [
+    (4, 128, 96, 16, [1, 5, 64, 130, 203], [1, 3, 64, 1, 17]),
+    (16, 576, 512, 16, [700, 1500], [1, 1]),                # single tokens: the keys cut into chunks
+    (16, 576, 512, 16, [300, 77], [300, 77]),               # whole prompts
+    (2, 128, 64, 8, [1100, 17, 2], [300, 17, 2]),
+    (40, 96, 32, 4, [150, 1], [9, 1]),                      # more heads than a tile has columns
+    (12, 320, 256, 32, [900], [33]),
+    (1, 48, 32, 16, [70, 200], [70, 1]),
+])
+def test_many_heads_on_one_wide_key_value_head(ops16, H, DK, C, page, lengths, q_lens):
+    """What attention through latents asks of the attention kernels: every head reads the same key rows (wider than the
+    value rows). The matrix-core kernel against float64 and against the plain kernel on the same cache; the last query of
+    each long request is made to look at a key far back and at one at a page's last place."""
+    rng = np.random.default_rng(H + DK + sum(lengths))
+    ks, vs, cache, table = paged_rows(rng, lengths, DK, C, page, torch.bfloat16)
+    scale = 1.0 / math.sqrt(DK)
+    qs, positions, slots = [], [], []
+    for s, (n, ql) in enumerate(zip(lengths, q_lens)):
+        q = rng.standard_normal((ql, H, DK)).astype(np.float32)
+        if n > 100:
+            q[-1] += 5.0 * (ks[s][2] + ks[s][page - 1])[None, :] / math.sqrt(DK)
+        qs.append(q)
+        positions += list(range(n - ql, n))
+        slots += [s] * ql
+    q = dev(np.concatenate(qs).reshape(-1, H * DK), torch.bfloat16)
+    step = FakeStep(ints(positions), ints(slots), table, None)
+    out = torch.empty((q.shape[0], H * C), dtype=torch.bfloat16, device="cuda")
+    other = torch.empty_like(out)
+    ops16.paged_attention(q, H, 1, DK, cache, step, 0, scale, out, v_head_dim=C)
+    ops16.force_plain_attention = True
+    try:
+        ops16.paged_attention(q, H, 1, DK, cache, step, 0, scale, other, v_head_dim=C)
+    finally:
+        ops16.force_plain_attention = False
+    got, plain_got = out.float().cpu().numpy(), other.float().cpu().numpy()
+    assert np.max(np.abs(got - plain_got)) <= 0.03
+    at = 0
+    for s, (n, ql) in enumerate(zip(lengths, q_lens)):
+        k, v = rounded(ks[s], torch.bfloat16), rounded(vs[s], torch.bfloat16)
+        for i in sorted({0, ql // 2, ql - 1}):
+            p_ = n - ql + i
+            sc = (rounded(qs[s][i], torch.bfloat16) @ k[:p_ + 1].T) * scale
+            pr = np.exp(sc - sc.max(-1, keepdims=True))
+            want = ((pr / pr.sum(-1, keepdims=True)) @ v[:p_ + 1]).reshape(-1)
+            assert np.max(np.abs(got[at + i] - want)) <= 0.03, f"request {s} token {i}"
+        at += ql
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -1026,11 +1026,11 @@ def test_sampling_starts_without_waiting_for_the_stream(ops32, greedy):
 def test_kernels_refuse_what_they_cannot_do(ops32):
     from hf_cpu_amd.status import EngineError
     with pytest.raises(EngineError, match="head_dim"):
-        cache = FakeCache(group=0, k=torch.zeros((16, 512), device="cuda"), v=torch.zeros((16, 512), device="cuda"),
+        cache = FakeCache(group=0, k=torch.zeros((16, 1024), device="cuda"), v=torch.zeros((16, 1024), device="cuda"),
                           page_tokens=16, window=0)
         step = FakeStep(ints([0]), ints([0]), ints(np.zeros((1, 4))), None)
-        ops32.paged_attention(torch.zeros((1, 512), device="cuda"), 1, 1, 512, cache, step, 0, 1.0,
-                              torch.zeros((1, 512), device="cuda"))
+        ops32.paged_attention(torch.zeros((1, 1024), device="cuda"), 1, 1, 1024, cache, step, 0, 1.0,
+                              torch.zeros((1, 1024), device="cuda"))
     with pytest.raises(EngineError, match="shapes"):
         ops32.gemm(torch.zeros((2, 3), device="cuda"), torch.zeros((4, 5), device="cuda"),
                    torch.zeros((2, 4), device="cuda"))
