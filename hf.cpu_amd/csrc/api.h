@@ -217,8 +217,10 @@ int hfa_gate_mul(const void* x, int x_dtype, int ldx, const void* gate, int gate
 // latent before its norm, then the rotated key part) and `q` ([T, H (D + R)], head by head [D unrotated | R to be rotated]) it
 // writes packed[t] = [H heads of (R | C: left alone) | R | C | C]: the queries' parts to be rotated, the key's part to be rotated,
 // and the latent c = down[:C] / sqrt(mean(down[:C]^2) + eps) * w twice (as the key's rest and as the value). Sums in fp32.
+// `folded` ([T, H C] of q's type, or null): the heads' C parts are copied from there (else they are left alone).
 int hfa_latent_pack(const float* down, int ld_down, const void* q, int q_dtype, int ldq, const float* w, float eps, void* packed,
-                    int out_dtype, int ld_packed, int n_tokens, int n_heads, int dim, int rot, int latent, hipStream_t stream);
+                    int out_dtype, int ld_packed, int n_tokens, int n_heads, int dim, int rot, int latent, const void* folded,
+                    int ld_folded, hipStream_t stream);
 
 // hfa_channel_scan (recurrent.hip): per head, S [qk_dim][v_dim] in hfa_linear_scan's layout: S <- diag(a_t) S + k_t v_t^T, y_t = S^T
 // (q_scale q_t), with a decay per key channel formed in fp32 from gate[t, h qk_dim + n] + gate_bias[h qk_dim + n] = z:

@@ -308,8 +308,8 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
             for (int r = 0; r < 16; r++) {
                 const int kr = key0 + 8 * (r / 4) + 4 * half + (r % 4);
                 float sv = st[r] * sc;
-                if (softcap > 0.f) sv = softcap * (1.0f - 2.0f / (1.0f + fast_exp2(sv * cap2)));
-                st[r] = (kr >= vlo && kr <= vhi) ? 1.0f / (1.0f + fast_exp2(-1.4426950408889634f * (sv + hb))) : 0.f;
+                if (softcap > 0.f) sv = softcap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + fast_exp2(sv * cap2)));
+                st[r] = (kr >= vlo && kr <= vhi) ? __builtin_amdgcn_rcpf(1.0f + fast_exp2(-1.4426950408889634f * (sv + hb))) : 0.f;
             }
         } else {
             const bool inside = __all(!col_ok || (key0 >= vlo && key0 + KB - 1 <= vhi)) != 0;
@@ -745,8 +745,8 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
                     for (int r = 0; r < 16; r++) {
                         const int kr = key0 + 8 * (r / 4) + 4 * half + (r % 4);
                         float sv = st[r] * sc;
-                        if (softcap > 0.f) sv = softcap * (1.0f - 2.0f / (1.0f + fast_exp2(sv * cap2)));
-                        st[r] = (kr >= vlo && kr <= vhi) ? 1.0f / (1.0f + fast_exp2(-1.4426950408889634f * (sv + hb))) : 0.f;
+                        if (softcap > 0.f) sv = softcap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + fast_exp2(sv * cap2)));
+                        st[r] = (kr >= vlo && kr <= vhi) ? __builtin_amdgcn_rcpf(1.0f + fast_exp2(-1.4426950408889634f * (sv + hb))) : 0.f;
                     }
                 } else {
                     const bool inside = __all(!col_ok || (key0 >= vlo && key0 + KB - 1 <= vhi)) != 0;

@@ -980,13 +980,51 @@ class Ops:
                                           out.data_ptr(), _code(out), _rows(out, "gate_mul out"), x.shape[0], x.shape[1],
                                           self.ACTIVATIONS[kind], self._stream()))
 
-    def latent_pack(self, down, q, weight, eps, packed, n_heads, dim, rot, latent):
+    def head_products(self, a, w, out, n_heads):
+        """``out[t * H + h, :] = w[h] @ a[t * H + h, :K]``: a product per head, every head with a matrix of its own. ``a`` is
+        ``[T * H, >= K]`` (the heads' rows of all tokens, a token's heads one after the other), ``w`` ``[H, N, K]`` and ``out``
+        ``[T * H, >= N]``; both are usually views of ``[T, H * width]`` matrices. The heads are the experts of the grouped product
+        that the mixture of experts runs (``hfa_moe_plan``, ``hfa_moe_gemm``): one launch for all heads, on the matrix cores
+        where the sizes allow."""
+        self.settle()
+        self._whole(a)
+        self._scaled.pop(out.data_ptr(), None)
+        R, H = a.shape[0], int(n_heads)
+        if w.dim() != 3 or not w.is_contiguous() or w.shape[0] != H or R % H or out.shape[0] != R or a.shape[1] < w.shape[2] \
+                or out.shape[1] < w.shape[1] or (w.dtype != a.dtype and w.dtype != torch.float32):
+            fail(EINVAL, "head_products: a [T * heads, >= K], w [heads, N, K] contiguous, out [T * heads, >= N]")
+        N, K = int(w.shape[1]), int(w.shape[2])
+        code, wcode = _code(a), _code(w)
+        plain = 1 if self.force_plain_gemm else 0
+        tile_rows = 32 if plain else int(self.lib.hfa_moe_tile_rows(code, wcode, R, H, N, K))
+        max_tiles = R // tile_rows + H
+        key = ("head ids", H)
+        ids = self._shared.get(key)
+        if ids is None or ids.shape[0] * H < R:           # head h is the h-th choice of every token
+            if torch.cuda.is_current_stream_capturing():
+                fail(EINVAL, "head_products: the table of heads would have to grow while a graph is being captured")
+            rows = max(1024, 2 * (R // H))
+            ids = memory.to_device(torch.arange(H, dtype=torch.int32).repeat(rows, 1), self.device, "the heads as choices of every token")
+            self._shared[key] = ids
+        row_pair = self.scratch("heads_row_pair", (R,), torch.int32)
+        tiles = self.scratch("heads_tiles", (3 * max_tiles + 1,), torch.int32)
+        n_tiles = tiles[3 * max_tiles:]
+        self._check(self.lib.hfa_moe_plan(ids.data_ptr(), R, H, tile_rows, row_pair.data_ptr(), tiles.data_ptr(), n_tiles.data_ptr(),
+                                          self._stream()))
+        self._check(self.lib.hfa_moe_gemm(a.data_ptr(), _rows(a, "head rows"), code, 1, w.data_ptr(), wcode, row_pair.data_ptr(),
+                                          tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, tile_rows, out.data_ptr(), _rows(out, "head out"),
+                                          _code(out), 1, None, 0, N, K, plain, 0, 0.0, 0.0, 0.0, self._stream()))
+
+    def latent_pack(self, down, q, weight, eps, packed, n_heads, dim, rot, latent, folded=None):
         """The rows that ``rope_store`` and ``paged_attention`` take for attention through latents with one key/value head
         (key ``[rotated part | latent]``, value the latent): from ``down`` (fp32 [T, latent + rot]: the latent before its norm, then
         the key's part to be rotated) and ``q`` ([T, heads * (dim + rot)], a head being ``[dim | rot]``) it writes
-        ``packed[t] = [heads x (rot | latent: left alone) | rot | latent | latent]``, the latent RMS-normed with ``weight``."""
+        ``packed[t] = [heads x (rot | latent: left alone) | rot | latent | latent]``, the latent RMS-normed with ``weight``. ``folded``
+        (``[T, heads * latent]``): the heads' queries with the keys' expansion folded in, copied into the heads' latent parts."""
         self.settle()
         self._whole(q)
+        if folded is not None and (folded.shape[0] != down.shape[0] or folded.shape[1] < n_heads * latent or folded.dtype != q.dtype):
+            fail(EINVAL, "latent_pack: the folded queries are [T, heads * latent] of the queries' dtype")
         T = down.shape[0]
         if down.dtype != torch.float32 or down.shape[1] < latent + rot or q.shape[0] != T or q.shape[1] < n_heads * (dim + rot) \
                 or packed.shape[0] != T or packed.shape[1] < n_heads * (rot + latent) + rot + 2 * latent \
@@ -994,7 +1032,8 @@ class Ops:
             fail(EINVAL, "latent_pack: rows of the latent and the rotated part (fp32), the heads' queries, an fp32 weight of the latent's size")
         self._check(self.lib.hfa_latent_pack(down.data_ptr(), _rows(down, "latent rows"), q.data_ptr(), _code(q), _rows(q, "queries"),
                                              weight.data_ptr(), float(eps), packed.data_ptr(), _code(packed), _rows(packed, "packed rows"),
-                                             T, n_heads, dim, rot, latent, self._stream()))
+                                             T, n_heads, dim, rot, latent, None if folded is None else folded.data_ptr(),
+                                             0 if folded is None else _rows(folded, "folded queries"), self._stream()))
 
     # ---- layer norm, plain activations, soft cap -----------------------------------------------------------------
     def layernorm(self, x, weight, bias, eps, out, rows=None):

@@ -372,18 +372,19 @@ class LatentAttention(Part):
             ops.group_rmsnorm(down[:, :rq], self.q_norm_w, self.eps, 1, cq)
             ops.gemm(cq, self.w_uq, q)
         packed = ops.scratch("qkv", (T, H * HD + HD + C), ops.act_dtype)
+        folded = ops.scratch("latent_q_folded", (T, H * C), ops.act_dtype)
         with ops.section("latent_pack"):
-            ops.latent_pack(down[:, rq:], q, self.kv_norm_w, self.eps, packed, H, D, R, C)
-            for hd in range(H):                  # the keys' expansion, folded into each head's query
-                ops.gemm(q[:, hd * (D + R):hd * (D + R) + D], self.w_uk_t[hd], packed[:, hd * HD + R:(hd + 1) * HD])
+            # the keys' expansion, folded into each head's query: one grouped product over the heads
+            ops.head_products(q.view(T * H, D + R), self.w_uk_t, folded.view(T * H, C), H)
+            ops.latent_pack(down[:, rq:], q, self.kv_norm_w, self.eps, packed, H, D, R, C, folded=folded)
             self.position.store(ops, step, packed, H, 1, cache, True, v_head_dim=C)
         att = ops.scratch("latent_att", (T, H * C), ops.act_dtype)
         with ops.section("latent_attn"):
             ops.paged_attention(packed, H, 1, HD, cache, step, 0, self.scale, att, v_head_dim=C)
         heads = ops.scratch("att", (T, H * Dv), ops.act_dtype)
         with ops.section("latent_v"):
-            for hd in range(H):                  # the values' expansion of each head's weighted sum of latents
-                ops.gemm(att[:, hd * C:(hd + 1) * C], self.w_uv[hd * Dv:(hd + 1) * Dv], heads[:, hd * Dv:(hd + 1) * Dv])
+            # the values' expansion of each head's weighted sum of latents
+            ops.head_products(att.view(T * H, C), self.w_uv.view(H, Dv, C), heads.view(T * H, Dv), H)
             if self.out_gate:
                 ops.gate_mul(heads, gate, heads, "sigmoid")
         with ops.section("latent_wo"):
