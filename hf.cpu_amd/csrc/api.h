@@ -223,14 +223,15 @@ int hfa_latent_pack(const float* down, int ld_down, const void* q, int q_dtype, 
                     int ld_folded, hipStream_t stream);
 
 // hfa_channel_scan (recurrent.hip): per head, S [qk_dim][v_dim] in hfa_linear_scan's layout: S <- diag(a_t) S + k_t v_t^T, y_t = S^T
-// (q_scale q_t), with a decay per key channel formed in fp32 from gate[t, h qk_dim + n] + gate_bias[h qk_dim + n] = z:
-// form 0: a = lower[h qk_dim + n] + (1 - lower) sigmoid(z), and k_t = 1 - a_t (k is not read);
-// form 1: a = sigmoid(z)^inv_tau = exp(inv_tau logsigmoid(z)), k_t read from k.
-// q_act HFA_ACT_SILU: the queries pass silu first (0: as they are).
-int hfa_channel_scan(const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, int dtype, const void* gate,
-                     int gate_dtype, int ld_gate, const float* gate_bias, int form, const float* lower, float inv_tau, int q_act,
-                     int n_heads, int qk_dim, int v_dim, float q_scale, float* state, size_t state_ld, const int* q_start,
-                     const int* seq_slot, int n_seqs, float* y, int ldy, hipStream_t stream);
+// (q_scale q_t), with a decay per key channel a_t = decay[t, h qk_dim + n] (fp32); kcomp 1: k_t = 1 - a_t (k is not read), else k_t
+// is read from k. q_act HFA_ACT_SILU: the queries pass silu first (0: as they are). hfa_channel_decay forms the decays in fp32 from
+// x = z[r, c] + bias[c] (bias null: 0): form 0: a = lower[c] + (1 - lower[c]) sigmoid(x); form 1: a = sigmoid(x)^inv_tau =
+// exp(inv_tau logsigmoid(x)).
+int hfa_channel_decay(const void* z, int z_dtype, int ldz, const float* bias, int form, const float* lower, float inv_tau,
+                      float* out, int ldo, int n_rows, int width, hipStream_t stream);
+int hfa_channel_scan(const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, int dtype, const float* decay,
+                     int ld_decay, int kcomp, int q_act, int n_heads, int qk_dim, int v_dim, float q_scale, float* state,
+                     size_t state_ld, const int* q_start, const int* seq_slot, int n_seqs, float* y, int ldy, hipStream_t stream);
 
 // out[r, c] = act(in[r, c]) for rows of `width` values with strides ldi and ldo, computed in fp32:
 // the exact gelu 0.5 z (1 + erf(z / sqrt 2)), its tanh form, relu(z)^2, silu or the logistic function.

@@ -607,19 +607,16 @@ extern "C" int hfa_delta_scan(const float* q, int ldq, const float* k, int ldk, 
 }
 
 // ---- a decay per key channel -------------------------------------------------------------------------------------------
-// Per head, S [N][P] in the state row, in hfa_linear_scan's layout: S <- diag(a_t) S + k_t v_t^T, y_t = S^T (q_scale q_t). The
-// decays are formed here, in fp32, from z = gate[t, h N + n] + gate_bias[h N + n]:
-//   form 0: a = lower[h N + n] + (1 - lower[h N + n]) sigmoid(z), and the key is the decay's complement, k = 1 - a (a forget gate
-//           that also decides what is written; no keys are read);
-//   form 1: a = sigmoid(z)^inv_tau, as exp(inv_tau logsigmoid(z)); keys are read.
-// q_act HFA_ACT_SILU: the queries pass silu on their way in. The block, its lanes and the staging through LDS are
-// linear_scan_kernel's, with the decays staged beside the keys as delta_scan_kernel stages its own; nothing crosses lanes
-// inside the walk.
-template <typename T, typename TG, int NS, int NPT>
+// Per head, S [N][P] in the state row, in hfa_linear_scan's layout: S <- diag(a_t) S + k_t v_t^T, y_t = S^T (q_scale q_t), with
+// the decays a_t[n] given in fp32 ([T, H N], formed beforehand by hfa_channel_decay: every block of a head's columns would
+// otherwise form the same decays again). kcomp 1: the key is the decay's complement, k = 1 - a (a forget gate that also decides
+// what is written; no keys are read); else keys are read. q_act HFA_ACT_SILU: the queries pass silu on their way in. The block,
+// its lanes and the staging through LDS are linear_scan_kernel's, with the decays staged beside the keys as delta_scan_kernel
+// stages its own; nothing crosses lanes inside the walk.
+template <typename T, int NS, int NPT>
 __global__ __launch_bounds__(SCAN_THREADS) void channel_scan_kernel(
     const T* __restrict__ q, int ldq, const T* __restrict__ k, int ldk, int N, const T* __restrict__ v, int ldv, int P,
-    const TG* __restrict__ gate, int ld_gate, const float* __restrict__ gate_bias, int form, const float* __restrict__ lower,
-    float inv_tau, int q_act, float q_scale, float* __restrict__ state, size_t state_ld, const int* __restrict__ q_start,
+    const float* __restrict__ decay, int ld_decay, int kcomp, int q_act, float q_scale, float* __restrict__ state, size_t state_ld, const int* __restrict__ q_start,
     const int* __restrict__ seq_slot, float* __restrict__ y, int ldy) {
     constexpr int NPAD = NS * NPT, PT = SCAN_THREADS / NS, TOK = SCAN_TOKENS;
     constexpr int RK = TOK * NPAD / SCAN_THREADS, RV = (TOK * PT + SCAN_THREADS - 1) / SCAN_THREADS;
@@ -640,15 +637,8 @@ __global__ __launch_bounds__(SCAN_THREADS) void channel_scan_kernel(
     for (int i = 0; i < NPT; i++) st[i] = S[(size_t)i * p_pad * NS];
     const T* kg = k ? k + (size_t)q0 * ldk + h * N : nullptr;
     const T* qg = q + (size_t)q0 * ldq + h * N;
-    const TG* gg = gate + (size_t)q0 * ld_gate + h * N;
+    const float* gg = decay + (size_t)q0 * ld_decay + h * N;
     const T* vg = v + (size_t)q0 * ldv + h * P + pz * PT;
-    float bias_r[RK], lower_r[RK];                         // of the channels this thread stages
-#pragma unroll
-    for (int r = 0; r < RK; r++) {
-        const int n = (tid + r * SCAN_THREADS) % NPAD;
-        bias_r[r] = (n < N && gate_bias) ? gate_bias[h * N + n] : 0.f;
-        lower_r[r] = (n < N && form == 0) ? lower[h * N + n] : 0.f;
-    }
     struct Staged { float k[RK], q[RK], z[RK], v[RV]; };
     Staged set_a, set_b;
     auto fetch = [&](Staged& g_, int c0) {
@@ -657,9 +647,9 @@ __global__ __launch_bounds__(SCAN_THREADS) void channel_scan_kernel(
         for (int r = 0; r < RK; r++) {
             const int idx = tid + r * SCAN_THREADS, t = c0 + idx / NPAD, n = idx % NPAD;
             const bool ok = t < n_tok && n < N;
-            g_.k[r] = (ok && form == 1) ? to_f32(kg[(size_t)t * ldk + n]) : 0.f;
+            g_.k[r] = (ok && !kcomp) ? to_f32(kg[(size_t)t * ldk + n]) : 0.f;
             g_.q[r] = ok ? to_f32(qg[(size_t)t * ldq + n]) : 0.f;
-            g_.z[r] = ok ? to_f32(gg[(size_t)t * ld_gate + n]) : 0.f;
+            g_.z[r] = ok ? gg[(size_t)t * ld_decay + n] : 0.f;
         }
 #pragma unroll
         for (int r = 0; r < RV; r++) {
@@ -671,16 +661,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void channel_scan_kernel(
 #pragma unroll
         for (int r = 0; r < RK; r++) {
             const int idx = tid + r * SCAN_THREADS, n = idx % NPAD;
-            const float z = g_.z[r] + bias_r[r];
-            float a, kk;
-            if (form == 0) {
-                a = lower_r[r] + (1.0f - lower_r[r]) * (1.0f / (1.0f + expf(-z)));
-                kk = 1.0f - a;
-            } else {
-                const float ls = -(fmaxf(-z, 0.f) + log1pf(expf(-fabsf(z))));       // logsigmoid, exact for every z
-                a = expf(inv_tau * ls);
-                kk = g_.k[r];
-            }
+            const float a = g_.z[r], kk = kcomp ? 1.0f - a : g_.k[r];
             const bool live = n < N;                       // rows beyond N stay zero
             g_s[idx] = live ? a : 0.f;
             k_s[idx] = live ? kk : 0.f;
@@ -766,42 +747,71 @@ __global__ __launch_bounds__(SCAN_THREADS) void channel_scan_kernel(
     for (int i = 0; i < NPT; i++) S[(size_t)i * p_pad * NS] = st[i];
 }
 
-extern "C" int hfa_channel_scan(const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, int dtype, const void* gate,
-                                int gate_dtype, int ld_gate, const float* gate_bias, int form, const float* lower, float inv_tau,
-                                int q_act, int n_heads, int qk_dim, int v_dim, float q_scale, float* state, size_t state_ld,
-                                const int* q_start, const int* seq_slot, int n_seqs, float* y, int ldy, hipStream_t stream) {
-    HFA_REQUIRE(q && v && gate && state && q_start && seq_slot && y && n_seqs > 0, "channel_scan: a null argument");
+// The decays of hfa_channel_scan, in fp32, from x = z[r, c] + bias[c] (bias null: 0):
+//   form 0: a = lower[c] + (1 - lower[c]) sigmoid(x)                                 (a forget gate with a lower bound)
+//   form 1: a = sigmoid(x)^inv_tau, as exp(inv_tau logsigmoid(x))                    (a root of a sigmoid)
+template <typename TG>
+__global__ void channel_decay_kernel(const TG* __restrict__ z, int ldz, const float* __restrict__ bias, int form, const float* __restrict__ lower,
+                                     float inv_tau, float* __restrict__ out, int ldo, int width, size_t total) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t r = i / width, c = i % width;
+        const float x = to_f32(z[r * ldz + c]) + (bias ? bias[c] : 0.f);
+        float a;
+        if (form == 0) {
+            const float lo = lower[c];
+            a = lo + (1.0f - lo) * (1.0f / (1.0f + expf(-x)));
+        } else {
+            const float ls = -(fmaxf(-x, 0.f) + log1pf(expf(-fabsf(x))));       // logsigmoid, exact for every x
+            a = expf(inv_tau * ls);
+        }
+        out[r * ldo + c] = a;
+    }
+}
+
+extern "C" int hfa_channel_decay(const void* z, int z_dtype, int ldz, const float* bias, int form, const float* lower, float inv_tau,
+                                 float* out, int ldo, int n_rows, int width, hipStream_t stream) {
+    HFA_REQUIRE(z && out && n_rows > 0 && width > 0 && ldz >= width && ldo >= width, "channel_decay: bad arguments");
+    HFA_REQUIRE((form == 0 && lower) || (form == 1 && inv_tau > 0.f), "channel_decay: form 0 needs lower bounds, form 1 a positive 1 / tau");
+    HFA_REQUIRE(z_dtype == HFA_F32 || z_dtype == HFA_BF16, "channel_decay: unknown dtype %d", z_dtype);
+    const size_t total = (size_t)n_rows * width;
+    const int blocks = (int)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
+    if (z_dtype == HFA_F32) channel_decay_kernel<float><<<blocks, 256, 0, stream>>>((const float*)z, ldz, bias, form, lower, inv_tau, out, ldo, width, total);
+    else channel_decay_kernel<bf16><<<blocks, 256, 0, stream>>>((const bf16*)z, ldz, bias, form, lower, inv_tau, out, ldo, width, total);
+    HFA_LAUNCH_CHECK("channel_decay");
+    return 0;
+}
+
+extern "C" int hfa_channel_scan(const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, int dtype, const float* decay,
+                                int ld_decay, int kcomp, int q_act, int n_heads, int qk_dim, int v_dim, float q_scale, float* state,
+                                size_t state_ld, const int* q_start, const int* seq_slot, int n_seqs, float* y, int ldy, hipStream_t stream) {
+    HFA_REQUIRE(q && v && decay && state && q_start && seq_slot && y && n_seqs > 0 && (kcomp || k), "channel_scan: a null argument");
     HFA_REQUIRE(n_heads > 0 && qk_dim > 0 && v_dim > 0, "channel_scan: bad sizes");
-    HFA_REQUIRE((form == 0 && lower) || (form == 1 && k && inv_tau > 0.f),
-                "channel_scan: form 0 needs the decays' lower bounds, form 1 keys and a positive 1 / tau");
     HFA_REQUIRE(q_act == HFA_ACT_NONE || q_act == HFA_ACT_SILU, "channel_scan: the queries pass silu or nothing");
     HFA_REQUIRE(qk_dim <= 256, "channel_scan: a state of %d rows a head is too large (at most 256)", qk_dim);
-    HFA_REQUIRE(ldq >= n_heads * qk_dim && (form == 0 || ldk >= n_heads * qk_dim) && ldv >= n_heads * v_dim && ldy >= n_heads * v_dim &&
-                    ld_gate >= n_heads * qk_dim && state_ld >= hfa_linear_scan_state_floats(n_heads, qk_dim, v_dim),
+    HFA_REQUIRE(ldq >= n_heads * qk_dim && (kcomp || ldk >= n_heads * qk_dim) && ldv >= n_heads * v_dim && ldy >= n_heads * v_dim &&
+                    ld_decay >= n_heads * qk_dim && state_ld >= hfa_linear_scan_state_floats(n_heads, qk_dim, v_dim),
                 "channel_scan: a row is shorter than its heads (a state row holds hfa_linear_scan_state_floats values)");
-    HFA_REQUIRE((dtype == HFA_F32 || dtype == HFA_BF16) && (gate_dtype == HFA_F32 || gate_dtype == HFA_BF16) &&
-                    !(dtype == HFA_F32 && gate_dtype == HFA_BF16), "channel_scan: unknown mix of dtypes");
+    HFA_REQUIRE(dtype == HFA_F32 || dtype == HFA_BF16, "channel_scan: unknown dtype %d", dtype);
     int ns, npt;
     scan_shape(qk_dim, &ns, &npt);
     const int pt = SCAN_THREADS / ns, p_tiles = (v_dim + pt - 1) / pt;
     HFA_REQUIRE(n_heads <= 65535 && n_seqs <= 65535 && p_tiles <= 65535, "channel_scan: the step exceeds the grid");
     dim3 grid(n_heads, n_seqs, p_tiles);
-#define CH_GO(T, TG, NS, NPT)                                                                                              \
-    channel_scan_kernel<T, TG, NS, NPT><<<grid, SCAN_THREADS, 0, stream>>>(                                                \
-        (const T*)q, ldq, (const T*)k, ldk, qk_dim, (const T*)v, ldv, v_dim, (const TG*)gate, ld_gate, gate_bias, form, lower, \
-        inv_tau, q_act, q_scale, state, state_ld, q_start, seq_slot, y, ldy)
-#define CH_SIZES(T, TG)                                          \
-    do {                                                         \
-        if (ns == 4) CH_GO(T, TG, 4, 4);                         \
-        else if (ns == 8 && npt == 4) CH_GO(T, TG, 8, 4);        \
-        else if (ns == 8) CH_GO(T, TG, 8, 8);                    \
-        else if (npt == 4) CH_GO(T, TG, 16, 4);                  \
-        else if (npt == 8) CH_GO(T, TG, 16, 8);                  \
-        else CH_GO(T, TG, 16, 16);                               \
+#define CH_GO(T, NS, NPT)                                                                                                      \
+    channel_scan_kernel<T, NS, NPT><<<grid, SCAN_THREADS, 0, stream>>>((const T*)q, ldq, (const T*)k, ldk, qk_dim, (const T*)v, ldv, v_dim, \
+                                                                       decay, ld_decay, kcomp, q_act, q_scale, state, state_ld, q_start,  \
+                                                                       seq_slot, y, ldy)
+#define CH_SIZES(T)                                          \
+    do {                                                     \
+        if (ns == 4) CH_GO(T, 4, 4);                         \
+        else if (ns == 8 && npt == 4) CH_GO(T, 8, 4);        \
+        else if (ns == 8) CH_GO(T, 8, 8);                    \
+        else if (npt == 4) CH_GO(T, 16, 4);                  \
+        else if (npt == 8) CH_GO(T, 16, 8);                  \
+        else CH_GO(T, 16, 16);                               \
     } while (0)
-    if (dtype == HFA_F32) CH_SIZES(float, float);
-    else if (gate_dtype == HFA_F32) CH_SIZES(bf16, float);
-    else CH_SIZES(bf16, bf16);
+    if (dtype == HFA_F32) CH_SIZES(float);
+    else CH_SIZES(bf16);
 #undef CH_SIZES
 #undef CH_GO
     HFA_LAUNCH_CHECK("channel_scan");

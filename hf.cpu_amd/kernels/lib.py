@@ -25,7 +25,8 @@ _SIGNATURES = {
     "hfa_scale_add": [P, I, P, F, P, I, I, I, I, P],
     "hfa_gate_mul": [P, I, I, P, I, I, P, I, I, I, I, I, P],
     "hfa_latent_pack": [P, I, P, I, I, P, F, P, I, I, I, I, I, I, I, P, I, P],
-    "hfa_channel_scan": [P, I, P, I, P, I, I, P, I, I, P, I, P, F, I, I, I, I, F, P, c_size_t, P, P, I, P, I, P],
+    "hfa_channel_scan": [P, I, P, I, P, I, I, P, I, I, I, I, I, I, F, P, c_size_t, P, P, I, P, I, P],
+    "hfa_channel_decay": [P, I, I, P, I, P, F, P, I, I, I, P],
     "hfa_group_rmsnorm": [P, I, I, P, P, I, I, P, I, I, I, F, P, I, I, I, P, P],
     "hfa_delta_scan": [P, I, P, I, I, I, P, I, I, I, P, I, P, P, P, I, F, F, P, c_size_t, P, P, I, I, P, I, P],
     "hfa_embed_pos": [P, I, P, P, P, P, I, I, I, F, P],

@@ -934,8 +934,7 @@ class Ops:
         if (lower is None) == (tau is None) or (form == 1) != (k is not None):
             fail(EINVAL, "channel_scan: either lower bounds and no keys, or tau and keys")
         if q.dtype != v.dtype or (k is not None and k.dtype != q.dtype) or y.dtype != torch.float32 or state.dtype != torch.float32 \
-                or state.stride(1) != 1 or q.shape[0] != T or v.shape[0] != T or gate.shape[0] != T or y.shape[1] != n_heads * v_dim \
-                or (q.dtype == torch.float32 and gate.dtype != torch.float32):
+                or state.stride(1) != 1 or q.shape[0] != T or v.shape[0] != T or gate.shape[0] != T or y.shape[1] != n_heads * v_dim:
             fail(EINVAL, "channel_scan: q, k and v of one dtype and the step's rows, fp32 output and state")
         for t, what in ((gate_bias, "gate_bias"), (lower, "lower")):
             if t is not None and (t.dtype != torch.float32 or t.numel() != n_heads * qk_dim or not t.is_contiguous()):
@@ -947,12 +946,16 @@ class Ops:
 
         def ptr(t):
             return None if t is None else t.data_ptr()
+        # the decays once a (token, head, channel), not once more in every block of a head's columns
+        inv_tau = 0.0 if tau is None else 1.0 / float(tau)
+        decays = self.scratch("channel_decays", (T, n_heads * qk_dim), torch.float32)
+        self._check(self.lib.hfa_channel_decay(gate.data_ptr(), _code(gate), _rows(gate, "scan gate"), ptr(gate_bias), form, ptr(lower), inv_tau,
+                                               decays.data_ptr(), _rows(decays, "decays"), T, n_heads * qk_dim, self._stream()))
         self._check(self.lib.hfa_channel_scan(
             q.data_ptr(), _rows(q, "scan q"), ptr(k), 0 if k is None else _rows(k, "scan k"), v.data_ptr(), _rows(v, "scan v"), _code(q),
-            gate.data_ptr(), _code(gate), _rows(gate, "scan gate"), ptr(gate_bias), form, ptr(lower), 0.0 if tau is None else 1.0 / float(tau),
-            self.ACTIVATIONS["silu"] if q_act else 0, n_heads, qk_dim, v_dim, float(q_scale), state.data_ptr(), state.stride(0),
-            _ints(step.q_start, "q_start", step.n_seqs + 1), _ints(step.seq_slot, "seq_slot", step.n_seqs), step.n_seqs, y.data_ptr(),
-            _rows(y, "scan out"), self._stream()))
+            decays.data_ptr(), _rows(decays, "decays"), 1 if form == 0 else 0, self.ACTIVATIONS["silu"] if q_act else 0, n_heads, qk_dim,
+            v_dim, float(q_scale), state.data_ptr(), state.stride(0), _ints(step.q_start, "q_start", step.n_seqs + 1),
+            _ints(step.seq_slot, "seq_slot", step.n_seqs), step.n_seqs, y.data_ptr(), _rows(y, "scan out"), self._stream()))
 
     def scale_add(self, y, out, scale=1.0, columns=None, accumulate=True):
         """``out (+)= scale * columns * y`` in fp32, ``columns`` an fp32 vector with one factor a column (None: 1): a branch's
