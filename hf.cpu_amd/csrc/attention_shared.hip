@@ -106,22 +106,36 @@ __global__ __launch_bounds__(4 * WAVE) void attn_shared_kernel(
         for (int r = 0; r < 16; r++) o[j][r] = 0.f;
     float m = SH_NEG_BIG, l = 0.f;
 
-    int it = 0;
-    for (int key0 = (k_begin / SH_KB) * SH_KB; key0 <= k_end; key0 += SH_KB, it++) {
-        // this lane's row of the key block (rows past the end repeat the last key; they are masked)
-        ShFrag kf[KSW], vf[NDBW][2];
-        {
-            int key = key0 + col;
-            key = key < hi ? key : hi;
-            const size_t row = ((size_t)bt[key >> psh] << psh) + (key & (P - 1));
-            const uint16_t* kp = kc + row * DK + half * 8;
+    // this lane's row of a key block (rows past the end repeat the last key; they are masked)
+    auto load_k = [&](int key0, ShFrag (&kf)[KSW]) {
+        int key = key0 + col;
+        key = key < hi ? key : hi;
+        const size_t row = ((size_t)bt[key >> psh] << psh) + (key & (P - 1));
+        const uint16_t* kp = kc + row * DK + half * 8;
 #pragma unroll
-            for (int j = 0; j < KSW; j++) {
-                const int ks = wave + 4 * j;
-                kf[j].u = ks * 16 < DK ? *reinterpret_cast<const uint4*>(kp + ks * 16) : make_uint4(0, 0, 0, 0);
-            }
+        for (int j = 0; j < KSW; j++) {
+            const int ks = wave + 4 * j;
+            kf[j].u = ks * 16 < DK ? *reinterpret_cast<const uint4*>(kp + ks * 16) : make_uint4(0, 0, 0, 0);
         }
+    };
+    // The keys of the next block are asked for before this block's products begin, and this block's values as soon as its
+    // scores' partial sums are on their way to LDS: the trips to memory run beside the exchange, the softmax and the products.
+    int it = 0;
+    const int key_first = (k_begin / SH_KB) * SH_KB;
+    ShFrag kf[KSW], kn[KSW];
+    if (key_first <= k_end) load_k(key_first, kf);
+    for (int key0 = key_first; key0 <= k_end; key0 += SH_KB, it++) {
+        load_k(key0 + SH_KB <= k_end ? key0 + SH_KB : key0, kn);
+        sh_floatx16 st;
+#pragma unroll
+        for (int r = 0; r < 16; r++) st[r] = 0.f;
+#pragma unroll
+        for (int j = 0; j < KSW; j++) st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[j].v, qf[j].v, st, 0, 0, 0);
+        const int buf = it & 1;
+#pragma unroll
+        for (int r = 0; r < 16; r++) part_s[buf][wave][r][lane] = st[r];
         // values: for product step kk the lane needs keys key0 + 16 kk + 8 run + 4 half + {0..3} of dimension 32 db + col
+        ShFrag vf[NDBW][2];
 #pragma unroll
         for (int kk = 0; kk < 2; kk++)
 #pragma unroll
@@ -135,14 +149,6 @@ __global__ __launch_bounds__(4 * WAVE) void attn_shared_kernel(
                     vf[j][kk].h[run] = db * 32 < C ? *reinterpret_cast<const uint2*>(vp + ((size_t)(db * 32 + col) << psh)) : make_uint2(0, 0);
                 }
             }
-        sh_floatx16 st;
-#pragma unroll
-        for (int r = 0; r < 16; r++) st[r] = 0.f;
-#pragma unroll
-        for (int j = 0; j < KSW; j++) st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[j].v, qf[j].v, st, 0, 0, 0);
-        const int buf = it & 1;
-#pragma unroll
-        for (int r = 0; r < 16; r++) part_s[buf][wave][r][lane] = st[r];
         __syncthreads();
 #pragma unroll
         for (int r = 0; r < 16; r++)
@@ -157,10 +163,10 @@ __global__ __launch_bounds__(4 * WAVE) void attn_shared_kernel(
         }
         mx = sh_pair_max(mx);
         const float mn = fmaxf(m, mx);
-        const float corr = exp2f(m - mn);
+        const float corr = __builtin_amdgcn_exp2f(m - mn);
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-            const float p = st[r] > 0.5f * SH_NEG_BIG ? exp2f(st[r] - mn) : 0.f;
+            const float p = st[r] > 0.5f * SH_NEG_BIG ? __builtin_amdgcn_exp2f(st[r] - mn) : 0.f;
             st[r] = p;
             psum += p;
         }
@@ -208,6 +214,8 @@ __global__ __launch_bounds__(4 * WAVE) void attn_shared_kernel(
         for (int kk = 0; kk < 2; kk++)
 #pragma unroll
             for (int j = 0; j < NDBW; j++) o[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[j][kk].v, pf[kk].v, o[j], 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < KSW; j++) kf[j].u = kn[j].u;
     }
     if (!col_ok) return;
     // element r of o[j]: value dimension 32 (wave + 4 j) + 8 (r / 4) + 4 half + r % 4 of this lane's column

@@ -1007,6 +1007,8 @@ class Ops:
             if torch.cuda.is_current_stream_capturing():
                 fail(EINVAL, "head_products: the table of heads would have to grow while a graph is being captured")
             rows = max(1024, 2 * (R // H))
+            if ids is not None:                           # captured graphs may still read the smaller table: it stays alive
+                self._shared[key + (ids.shape[0],)] = ids
             ids = memory.to_device(torch.arange(H, dtype=torch.int32).repeat(rows, 1), self.device, "the heads as choices of every token")
             self._shared[key] = ids
         row_pair = self.scratch("heads_row_pair", (R,), torch.int32)

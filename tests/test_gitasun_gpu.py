@@ -659,6 +659,28 @@ def test_a_long_prompt_decoded_token_by_token(gpu, tmp_path, dtype):
     engine.manager.check()
 
 
+def test_graphs_of_decode_steps_survive_a_longer_prompt(gpu, tmp_path):
+    """Decode steps of a short request are captured into graphs; then a prompt arrives that is longer than anything before
+    (work buffers and the table of heads behind the heads' grouped products grow); the short request's next steps, replayed
+    or captured anew, still give the plain logits."""
+    import hf_cpu_amd
+    cfg = gh.config(120, 64, residual_mult=0.9, layers=[gh.layer(gh.latent(4, 16, 16, 16, 48, 24), gh.dense(64)),
+                                                        gh.layer(gh.hgrn2(2, 16, 16), None)])
+    d = gh.make_model_dir(str(tmp_path / "m"), cfg, seed=2, stored="BF16")
+    reqs = gh.random_requests(cfg, [40, 1300], seed=5)
+    want = gh.plain_logits(d, reqs)
+    a, b = reqs["r0"], reqs["r1"]
+    steps = [helpers._step(0, [("r0", a[:20], [19])])]
+    steps += [helpers._step(len(steps) + i, [("r0", a[20 + i:21 + i], [0])]) for i in range(8)]
+    steps.append(helpers._step(len(steps), [("r1", b, [0, 1299])], ["r1"]))
+    steps += [helpers._step(len(steps) + i, [("r0", a[28 + i:29 + i], [0])], ["r0"] if i == 11 else []) for i in range(12)]
+    for dtype in ("float32", "bfloat16"):
+        engine = hf_cpu_amd.load_engine(d, dtype=dtype, page_tokens=16, max_tokens=helpers.max_live_tokens(steps), max_seqs=2)
+        got = helpers.run_trace_in_engine(engine, steps)
+        assert engine.graph_replays > 0
+        compare_for(dtype, got, want, TOL[dtype], f"graphs and a longer prompt {dtype}")
+
+
 def test_random_weights_and_other_orders_of_layers(gpu, tmp_path):
     """``write_random_model`` makes a folder for this design too (the latents' and the decay's inner sizes from the
     configuration), and the engine reads it back: a model of one recurrence, one of one side-by-side layer with a single
