@@ -132,7 +132,7 @@ def gitasun_work(z, T, batch, ctx):
     L = 3 * n3
     params = {"latent_down": n3 * W * (Q + C + R + QD), "latent_q": n3 * Q * H * (D + R), "latent_pack": n3 * H * D * C, "latent_v": n3 * H * D * C,
               "latent_wo": n3 * QD * W, "qkv": n3 * W * (2 * QD + 2 * KD), "wo": n3 * QD * W, "forget_in": n3 * W * 3 * QD, "forget_wo": n3 * QD * W,
-              "gla_in": n3 * (W * (4 * QD + 16) + 16 * QD), "gla_wo": n3 * QD * W, "router": L * E * W, "shared_expert": L * 3 * F * W, "head": V * W}
+              "gla_in": n3 * (W * (4 * QD + 16) + 16 * QD), "gla_wo": n3 * QD * W, "router": L * E * W, "gate_up": L * 2 * F * W, "down": L * F * W, "head": V * W}      # (gate_up, down: the shared expert)
     pre = {k: 2.0 * T * v for k, v in params.items() if k != "head"}
     pre["latent_attn"] = n3 * 2.0 * (R + 2 * C) * H * T * (T + 1) / 2
     pre["attn"] = n3 * 4.0 * D * H * T * (T + 1) / 2
