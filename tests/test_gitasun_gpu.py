@@ -562,6 +562,42 @@ def test_greedy_generation_through_the_session(gpu, tiny):
             toks.append(t)
 
 
+def test_command_line_generates_and_forks(gpu, tiny):
+    """bin/hfamd on a folder of this design: greedy tokens are the plain implementation's; two continuations of one prompt
+    (the second forks the first's pages and state rows after the prompt) drawn with seeds of their own start from the same
+    logits; sampled runs with one seed repeat themselves."""
+    import os
+    import subprocess
+    import sys
+    name, cfg, d, reqs, _ = tiny
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    prompt = reqs["r3"]
+
+    def run(extra):
+        r = subprocess.run([sys.executable, os.path.join(root, "bin", "hfamd"), "--stdin-mode", "none", "--model", d, "--dtype", "float32",
+                            "--ctx-max", "128", "--page-size", str(gh.PAGE[name]), "--max-seqs", "4", "--log-level", "error",
+                            "--prompt-ids", " ".join(map(str, prompt))] + extra, text=True, capture_output=True, timeout=300)
+        assert r.returncode == 0, r.stderr
+        toks = {}
+        for line in r.stdout.replace("\x1e", "\n").splitlines():
+            if line.startswith("@token "):
+                f = dict(x.split("=", 1) for x in line.split(" ")[1:] if "=" in x)
+                toks.setdefault(f.get("seq", "0"), []).append(int(f["id"]))
+        return toks
+    greedy = run(["--temp", "0", "--max-tokens", "6"])["0"]
+    pcfg, w = pg.read_model(d)
+    toks = list(prompt)
+    for t in greedy:
+        row = pg.forward(pcfg, w, toks)[-1]
+        assert row[int(np.argmax(row))] - row[t] <= 1e-4 * max(1.0, float(np.max(np.abs(row))))
+        toks.append(t)
+    both = run(["--temp", "0", "--max-tokens", "5", "--n", "2"])
+    assert both["0"] == greedy[:5] and both["1"] == greedy[:5]
+    drawn = run(["--temp", "0.9", "--seed", "11", "--max-tokens", "8", "--n", "2"])
+    again = run(["--temp", "0.9", "--seed", "11", "--max-tokens", "8", "--n", "2"])
+    assert drawn == again and len(drawn["0"]) == 8 and len(drawn["1"]) == 8
+
+
 def far_key_model(kind):
     """One layer whose attention is made to look far back. The norm's output has (nearly) the stream's direction, the table's
     last two columns are zero but for token 1, whose entry in the column before the last is large, and for a constant last
