@@ -168,7 +168,7 @@ class GitasunConfig:
         if kind != "moe":
             fail(ENOTSUP, f"{f.origin}: a feed-forward of kind '{kind}' is not supported (supported: dense, moe)")
         router = cls._sub(f, "router")
-        experts = router.integer("experts", hi=256)
+        experts = router.integer("experts", hi=1024)
         top = router.integer("top", hi=64)
         if top > experts:
             fail(EFORMAT, f"{router.origin}: {top} choices among {experts} experts")
