@@ -252,26 +252,41 @@ __global__ __launch_bounds__(4 * WAVE) void attn_shared_kernel(
     }
 }
 
-// out[t, h, :] = sum_c o_c 2^(m_c - M) / sum_c l_c 2^(m_c - M), chunks in ascending order. One block a (token, head).
+// out[t, h, :] = sum_c o_c 2^(m_c - M) / sum_c l_c 2^(m_c - M), chunks in ascending order. One block a (token, head). The kernel is
+// a chain of trips to memory and little else: the chunks' maxima and sums are fetched by one thread each, at once, and a thread's
+// values of all chunks are asked for eight at a time before they are added.
 __global__ __launch_bounds__(256) void attn_shared_merge_kernel(const float* __restrict__ partial, uint16_t* __restrict__ out, int ldo, int H,
                                                                 int C, int n_chunks) {
-    __shared__ float w_s[SH_MAX_CHUNKS];
+    __shared__ float m_s[SH_MAX_CHUNKS], l_s[SH_MAX_CHUNKS], w_s[SH_MAX_CHUNKS];
     const int t = blockIdx.x, h = blockIdx.y;
     const size_t row = C + 2;
     const float* src = partial + (size_t)(t * H + h) * n_chunks * row;
+    if ((int)threadIdx.x < n_chunks) {
+        const float2 ml = *reinterpret_cast<const float2*>(src + threadIdx.x * row);
+        m_s[threadIdx.x] = ml.x;
+        l_s[threadIdx.x] = ml.y;
+    }
+    __syncthreads();
     float M = SH_NEG_BIG;
-    for (int c = 0; c < n_chunks; c++) M = fmaxf(M, src[c * row]);
+    for (int c = 0; c < n_chunks; c++) M = fmaxf(M, m_s[c]);
     float L = 0.f;
     for (int c = 0; c < n_chunks; c++) {
-        const float w = exp2f(src[c * row] - M);
+        const float w = exp2f(m_s[c] - M);
         if (threadIdx.x == 0) w_s[c] = w;
-        L = fmaf(src[c * row + 1], w, L);
+        L = fmaf(l_s[c], w, L);
     }
     __syncthreads();
     const float inv = 1.0f / L;
     for (int d = threadIdx.x; d < C; d += blockDim.x) {
         float acc = 0.f;
-        for (int c = 0; c < n_chunks; c++) acc = fmaf(src[c * row + 2 + d], w_s[c], acc);
+        for (int c0 = 0; c0 < n_chunks; c0 += 8) {
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) v[i] = c0 + i < n_chunks ? src[(c0 + i) * row + 2 + d] : 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                if (c0 + i < n_chunks) acc = fmaf(v[i], w_s[c0 + i], acc);
+        }
         out[(size_t)t * ldo + (size_t)h * C + d] = bf16_bits(acc * inv);
     }
 }
@@ -301,7 +316,7 @@ int attn_shared_launch(const AttnArgs& a, int v_head_dim) {
     const long blocks = (long)(one_each ? a.n_seqs : (a.n_tokens + tpt - 1) / tpt) * head_blocks;
     if (blocks < 512 && a.max_seq_len > 256 && a.workspace) {
         long want = (512 + blocks - 1) / blocks;
-        const long most = (a.max_seq_len + 127) / 128;
+        const long most = (a.max_seq_len + 127) / 128;        // no chunk of fewer than 128 keys (64 were measured: no gain)
         if (want > most) want = most;
         if (want > SH_MAX_CHUNKS) want = SH_MAX_CHUNKS;
         chunk_keys = (int)(((a.max_seq_len + want - 1) / want + SH_KB - 1) / SH_KB * SH_KB);
