@@ -113,10 +113,10 @@ def gitasun_shape(z):
                                                  rot=dict(dims=R, base=10000.0)), mlp=moe),
         dict(type="hgrn2", mixer=dict(heads=H, dim=D, vdim=D), mlp=moe),
         dict(type="parallel", mixer=dict(
-            left=dict(heads=H, kv_heads=G, dim=D, vdim=D, scale=1.0 / math.sqrt(D), softcap=30.0,
-                      rot=dict(dims=D, base=500000.0, scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192))),
-            right=dict(heads=H, dim=D, vdim=D, tau=16.0, decay_rank=16), left_scale=0.6, right_scale=1.1), mlp=moe)]
-    return dict(architecture="Gitasun", vocab=z["vocab"], width=W, embedding=dict(scale=math.sqrt(W)), residual_mult=0.7, norm=dict(eps=1e-6),
+            left=dict(heads=H, kv_heads=G, dim=D, vdim=D, scale=1.0 / math.sqrt(D), softcap=50.0,
+                      rot=dict(dims=D, base=500000.0, scaling=dict(factor=4.0, low=1.0, high=2.0, original=8192))),
+            right=dict(heads=H, dim=D, vdim=D, tau=8.0, decay_rank=16), left_scale=0.5, right_scale=1.0), mlp=moe)]
+    return dict(architecture="Gitasun", vocab=z["vocab"], width=W, embedding=dict(scale=math.sqrt(W)), residual_mult=0.5, norm=dict(eps=1e-6),
                 layers=three * z["triples"])
 
 

@@ -80,7 +80,7 @@ SMALL = config(131, 40, eps=1e-5, embedding_scale=3.0, residual_mult=0.8, layers
 CORES = config(520, 256, residual_mult=0.6, layers=[
     layer(latent(4, 64, 32, 64, 96, 128), moe(8, 2, 64, shared=128)),
     layer(hgrn2(4, 64, 64), dense(512)),
-    layer(parallel(left(8, 2, 64, 64, 32, base=50000.0, scaling=(8.0, 1.0, 4.0, 128), softcap=20.0), right(4, 32, 64, 8.0), 0.6, 1.1), moe(6, 3, 96)),
+    layer(parallel(left(8, 2, 64, 64, 32, base=40000.0, scaling=(6.0, 1.0, 3.0, 128), softcap=20.0), right(4, 32, 64, 8.0), 0.75, 1.25), moe(6, 3, 96)),
     layer(hgrn2(2, 128, 32), None),
     layer(latent(2, 32, 64, 128, 64, 64, base=1000.0), dense(256)),
     layer(parallel(left(4, 4, 32, 32, 32), right(2, 64, 128, 16.0), 1.0, 0.5), dense(320)),
@@ -202,10 +202,10 @@ def random_config(rng, big):
         else:
             G = pick(1, 2, 4)
             D = pick(32, 64, 128) if big else pick(6, 10, 16, 24)
-            lt = left(G * pick(1, 2, 3), G, D, D if big else pick(D, 4, 14), pick(D, D // 2 - (D // 2) % 2), base=pick(1000.0, 50000.0),
-                      scaling=pick(None, (8.0, 1.0, 4.0, 128)), softcap=pick(None, 10.0, 30.0))
-            rt = right(pick(1, 2, 4), pick(32, 64, 128) if big else pick(3, 8, 17, 24), pick(32, 64) if big else pick(4, 5, 12, 20), pick(1.0, 4.0, 16.0))
-            mix = parallel(lt, rt, pick(1.0, 0.6, -0.4), pick(1.0, 1.1, 0.3))
+            lt = left(G * pick(1, 2, 3), G, D, D if big else pick(D, 4, 14), pick(D, D // 2 - (D // 2) % 2), base=pick(1000.0, 40000.0),
+                      scaling=pick(None, (6.0, 1.0, 3.0, 128)), softcap=pick(None, 10.0, 25.0))
+            rt = right(pick(1, 2, 4), pick(32, 64, 128) if big else pick(3, 8, 17, 24), pick(32, 64) if big else pick(4, 5, 12, 20), pick(1.0, 4.0, 12.0))
+            mix = parallel(lt, rt, pick(1.0, 0.55, -0.4), pick(1.0, 1.15, 0.3))
         X = pick(2, 5, 8)
         ff = pick(None, dense(pick(32, 64, 96) if big else pick(4, 10, 24)),
                   moe(X, pick(1, 2, X), pick(32, 64, 96) if big else pick(4, 10, 32), shared=pick(None, 32 if big else 6)))

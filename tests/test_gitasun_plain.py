@@ -23,20 +23,21 @@ def test_tanh_gelu():
 
 
 def test_rescaled_frequencies():
-    base, dims = 50000.0, 48
+    base, dims = 30000.0, 40
     f = pg.rotary_frequencies(dims, base)
     assert np.allclose(f, [base ** (-2.0 * i / dims) for i in range(dims // 2)])
-    sc = dict(factor=8.0, low=1.0, high=4.0, original=512)
+    sc = dict(factor=6.0, low=1.0, high=3.0, original=256)
     g = pg.rotary_frequencies(dims, base, sc)
     wl = 2.0 * math.pi / f
-    assert np.array_equal(g[wl < 128.0], f[wl < 128.0]) and np.allclose(g[wl > 512.0], f[wl > 512.0] / 8.0)
-    mid = (wl >= 128.0) & (wl <= 512.0)
-    assert mid.any() and (wl < 128.0).any() and (wl > 512.0).any()
-    assert np.all(g[mid] <= f[mid]) and np.all(g[mid] >= f[mid] / 8.0)
+    short, long_ = 256 / 3.0, 256.0
+    assert np.array_equal(g[wl < short], f[wl < short]) and np.allclose(g[wl > long_], f[wl > long_] / 6.0)
+    mid = (wl >= short) & (wl <= long_)
+    assert mid.any() and (wl < short).any() and (wl > long_).any()
+    assert np.all(g[mid] <= f[mid]) and np.all(g[mid] >= f[mid] / 6.0)
     # the blend meets both ends: at l = original / high it is f, at l = original / low it is f / factor
-    for l_, want in ((128.0, 1.0), (512.0, 1.0 / 8.0)):
-        s = (512.0 / l_ - 1.0) / 3.0
-        assert math.isclose((1.0 - s) / 8.0 + s, want)
+    for l_, want in ((short, 1.0), (long_, 1.0 / 6.0)):
+        s = (256.0 / l_ - 1.0) / 2.0
+        assert math.isclose((1.0 - s) / 6.0 + s, want)
     assert np.allclose(pg.rotary_frequencies(dims, base, dict(sc, factor=1.0)), f, rtol=1e-14)
 
 
