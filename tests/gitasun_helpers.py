@@ -78,7 +78,7 @@ SMALL = config(131, 40, eps=1e-5, embedding_scale=3.0, residual_mult=0.8, layers
 # Sizes that the matrix-core kernels take: widths and heads that are multiples of 32, states of 64 x 64, 128 x 32, 32 x 64 and
 # 64 x 128, experts of 64 and 96.
 CORES = config(520, 256, residual_mult=0.6, layers=[
-    layer(latent(4, 64, 32, 64, 96, 128), moe(8, 2, 64, shared=128)),
+    layer(latent(4, 64, 32, 96, 96, 128), moe(8, 2, 64, shared=128)),
     layer(hgrn2(4, 64, 64), dense(512)),
     layer(parallel(left(8, 2, 64, 64, 32, base=40000.0, scaling=(6.0, 1.0, 3.0, 128), softcap=20.0), right(4, 32, 64, 8.0), 0.75, 1.25), moe(6, 3, 96)),
     layer(hgrn2(2, 128, 32), None),

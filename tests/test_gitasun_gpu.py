@@ -334,7 +334,7 @@ def test_many_heads_on_one_wide_key_value_head(ops16, H, DK, C, page, lengths, q
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,D,R,C", [(3, 6, 4, 10), (1, 8, 8, 5), (4, 64, 32, 96), (2, 32, 64, 64), (16, 128, 64, 512)])
+@pytest.mark.parametrize("H,D,R,C", [(3, 6, 4, 10), (1, 8, 8, 5), (4, 64, 64, 96), (2, 32, 64, 64), (16, 128, 64, 512)])
 def test_rows_for_attention_through_latents(ops32, dtype, H, D, R, C):
     rng = np.random.default_rng(H + D + C)
     T = 11
@@ -357,7 +357,7 @@ def test_rows_for_attention_through_latents(ops32, dtype, H, D, R, C):
     assert np.all(key[:, HD + C:] == 7.0)
 
 
-@pytest.mark.parametrize("E,top", [(5, 2), (12, 2), (4, 1), (3, 3), (64, 8), (256, 6)])
+@pytest.mark.parametrize("E,top", [(5, 2), (10, 2), (4, 1), (3, 3), (64, 8), (256, 6)])
 def test_router_with_the_softmax_over_the_chosen(ops32, E, top):
     rng = np.random.default_rng(E + top)
     T = 37
@@ -372,7 +372,7 @@ def test_router_with_the_softmax_over_the_chosen(ops32, E, top):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("W,F,E,top,T", [(40, 12, 5, 3, 9), (40, 32, 3, 3, 4), (256, 64, 8, 2, 70), (256, 96, 6, 3, 300), (128, 64, 12, 2, 1)])
+@pytest.mark.parametrize("W,F,E,top,T", [(40, 12, 5, 3, 9), (40, 32, 3, 3, 4), (256, 64, 8, 2, 70), (256, 96, 6, 3, 300), (128, 64, 10, 2, 1)])
 def test_gated_experts_weighted_on_their_output(ops32, ops16, dtype, W, F, E, top, T):
     """sum_e c_e Wdown_e (silu(Wgate_e h) * (Wup_e h)): the weight multiplies an expert's result, not its input."""
     ops = ops32 if dtype == torch.float32 else ops16
